@@ -44,10 +44,19 @@ class PrefixHit:
 def first_kept(rule, num_computed: int) -> int:
     """The first position whose keys a request still needs when its next token stands at `num_computed`. `rule`: an
     int (a trailing window of that many positions) or a tuple of ("window", n) / ("chunk", c) rules, the loosest of
-    which holds; a chunk rule keeps the block of c positions, counted from 0, that `num_computed` falls into."""
+    which holds; a chunk rule keeps the block of c positions, counted from 0, that `num_computed` falls into. A
+    ("first", n) entry is no rule of this kind (`pinned_prefix`)."""
     if isinstance(rule, int):
         return max(0, num_computed - rule + 1)
-    return min(max(0, num_computed - n + 1) if kind == "window" else (num_computed // n) * n for kind, n in rule)
+    return min(max(0, num_computed - n + 1) if kind == "window" else (num_computed // n) * n for kind, n in rule if kind != "first")
+
+
+def pinned_prefix(rule) -> int:
+    """How many positions from the request's start stay whatever the other rules have passed: the largest n of the
+    ("first", n) entries of a rule tuple, 0 without one."""
+    if rule is None or isinstance(rule, int):
+        return 0
+    return max([n for kind, n in rule if kind == "first"], default=0)
 
 
 class _Group:
@@ -89,7 +98,7 @@ class _Group:
 @dataclass
 class _Held:
     tables: list                                     # per group: page ids, -1 where given back
-    first_live: list                                 # per group: index of the first page still held
+    first_live: list                                 # per group: where the walk that gives pages back goes on
     state_slot: int = -1
     num_hashed: int = 0
 
@@ -199,7 +208,8 @@ class CacheManager:
             # the next tokens start at position num_computed and see keys from first_kept on
             first_needed = first_kept(g.window, num_computed)
             table = held.tables[gi]
-            i = held.first_live[gi]
+            # pages that hold one of the positions that stay for good are never given back: the walk starts behind them
+            i = max(held.first_live[gi], -(-pinned_prefix(g.window) // ps))
             while i < len(table) and (i + 1) * ps <= first_needed:
                 g.release(table[i])
                 table[i] = -1

@@ -521,3 +521,143 @@ class NegosunConfig:
     def flat(self) -> dict[str, Any]:
         return {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "num_hidden_layers": len(self.layers),
                 "experts": [None if layer.mlp is None else layer.mlp["experts"] for layer in self.layers]}
+
+
+# ------------------------------------------------------------------------------------ Tavevik
+
+@dataclass(frozen=True)
+class TavevikLayer:
+    """One entry of a Tavevik config's `layers`: the kind of its two-sided mixer, the sizes and constants of the left
+    (attention) and the right (recurrent) side with the optional keys resolved, the two output scales, and the
+    feed-forward's width and limit (None: the layer has no feed-forward)."""
+
+    kind: str                  # "parallel" or "parallel_2"
+    left: dict
+    right: dict
+    left_scale: float
+    right_scale: float
+    mlp: dict | None
+
+
+@register_config("Tavevik")
+@dataclass(frozen=True)
+class TavevikConfig:
+    """The ``config.json`` keys of the Tavevik design: layers whose mixer is softmax attention under a trailing window
+    beside a recurrence over a matrix per head, their outputs added under two scales; the norms sit on the sublayers'
+    outputs. Kind `parallel`: the attention keeps its first positions visible, bends its scores under a cap and gates
+    its heads element by element; the recurrence mixes each token's input with the previous token's and has a bonus for
+    the token itself. Kind `parallel_2`: the attention has biases and a sink per head; the recurrence is a delta rule
+    behind short convolutions. A feed-forward with a clamped gated activation; tied output weights. Every size and
+    constant comes from the file; the inner widths of the thin matrix pairs (`decay_rank`, `gate_rank`) come from the
+    checkpoint's tensors when the file does not name them."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: tuple
+    eos_token_id: int | None = None
+    max_position_embeddings: int | None = None
+
+    KINDS = ("parallel", "parallel_2")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, raw: dict[str, Any]) -> "TavevikConfig":
+        norm = raw.get("norm")
+        if not isinstance(norm, dict):
+            raise ConfigError("config.json lacks the object 'norm'")
+        listed = raw.get("layers")
+        if not isinstance(listed, list) or not listed:
+            raise ConfigError("config.json lacks the list 'layers'")
+        layers = []
+        for i, entry in enumerate(listed):
+            where = f"layers[{i}]"
+            kind = entry.get("type") if isinstance(entry, dict) else None
+            if kind not in cls.KINDS:
+                raise ConfigError(f"{where}: 'type' must be one of {list(cls.KINDS)}, got {kind!r}")
+            m = entry.get("mixer")
+            if not isinstance(m, dict) or not isinstance(m.get("left"), dict) or not isinstance(m.get("right"), dict):
+                raise ConfigError(f"{where} lacks the object 'mixer' with 'left' and 'right'")
+            l, r = m["left"], m["right"]
+            left = {key: _need(l, key, typ, where + ".mixer.left")
+                    for key, typ in (("heads", int), ("kv_heads", int), ("dim", int), ("vdim", int), ("scale", float))}
+            rot, mask = l.get("rot"), l.get("mask")
+            left["rot_dims"] = _need(rot, "dims", int, where + ".mixer.left.rot") if rot else 0
+            left["rot_base"] = _need(rot, "base", float, where + ".mixer.left.rot") if rot else 1.0
+            left["window"] = _need(mask, "size", int, where + ".mixer.left.mask") if mask else None
+            keep = mask.get("keep_first") if mask else None
+            left["keep_first"] = int(keep) if (keep and kind == "parallel") else 0
+            cap = l.get("softcap")
+            left["softcap"] = float(cap) if (cap and kind == "parallel") else None
+            right = {key: _need(r, key, int, where + ".mixer.right") for key in ("heads", "dim")}
+            right["decay_rank"] = r.get("decay_rank")
+            if kind == "parallel_2":
+                for key in ("kv_heads", "vdim", "conv"):
+                    right[key] = _need(r, key, int, where + ".mixer.right")
+                right["gate_rank"] = r.get("gate_rank")
+            mlp = entry.get("mlp")
+            ff = None
+            if mlp is not None:
+                if mlp.get("kind", "dense") != "dense":
+                    raise ConfigError(f"{where}.mlp: only kind 'dense' is known, got {mlp.get('kind')!r}")
+                ff = {"ff": _need(mlp, "ff", int, where + ".mlp"), "limit": _need(mlp, "limit", float, where + ".mlp")}
+            layers.append(TavevikLayer(kind, left, right, float(m.get("left_scale", 1.0)), float(m.get("right_scale", 1.0)), ff))
+        cfg = cls(vocab_size=_need(raw, "vocab", int), hidden_size=_need(raw, "width", int),
+                  norm_eps=_need(norm, "eps", float, "config.json norm"), layers=tuple(layers),
+                  eos_token_id=raw.get("eos_token_id"), max_position_embeddings=raw.get("max_position_embeddings"))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size < 1 or self.hidden_size < 1 or not self.norm_eps > 0:
+            raise ConfigError("vocab and width must be positive and norm.eps above zero")
+        for i, layer in enumerate(self.layers):
+            l, r, where = layer.left, layer.right, f"layers[{i}]"
+            if any(l[k] < 1 for k in ("heads", "kv_heads", "dim", "vdim")) or any(r[k] < 1 for k in r if isinstance(r[k], int)):
+                raise ConfigError(f"{where}: sizes must be positive")
+            if l["heads"] % l["kv_heads"]:
+                raise ConfigError(f"{where}: {l['heads']} heads are not a multiple of {l['kv_heads']} kv_heads")
+            if l["rot_dims"] % 2 or not 0 <= l["rot_dims"] <= l["dim"]:
+                raise ConfigError(f"{where}: rot.dims must be even and at most dim")
+            if l["window"] is not None and l["window"] < 1:
+                raise ConfigError(f"{where}: mask.size must be positive")
+            if l["keep_first"] < 0 or (l["keep_first"] and l["window"] is None):
+                raise ConfigError(f"{where}: mask.keep_first needs mask.size and must not be negative")
+            if l["softcap"] is not None and not l["softcap"] > 0:
+                raise ConfigError(f"{where}: softcap must be positive")
+            if layer.kind == "parallel_2" and r["heads"] % r["kv_heads"]:
+                raise ConfigError(f"{where}: the right side's {r['heads']} heads are not a multiple of its {r['kv_heads']} kv_heads")
+            if layer.mlp is not None and (layer.mlp["ff"] < 1 or not layer.mlp["limit"] > 0):
+                raise ConfigError(f"{where}.mlp: ff and limit must be positive")
+
+    def to_dict(self) -> dict[str, Any]:
+        """A ``config.json`` that reads back to an equal config."""
+        out = []
+        for layer in self.layers:
+            l = {k: layer.left[k] for k in ("heads", "kv_heads", "dim", "vdim", "scale")}
+            if layer.left["rot_dims"]:
+                l["rot"] = {"dims": layer.left["rot_dims"], "base": layer.left["rot_base"]}
+            if layer.left["window"] is not None:
+                l["mask"] = {"size": layer.left["window"]}
+                if layer.left["keep_first"]:
+                    l["mask"]["keep_first"] = layer.left["keep_first"]
+            if layer.left["softcap"] is not None:
+                l["softcap"] = layer.left["softcap"]
+            r = {k: v for k, v in layer.right.items() if v is not None}
+            mlp = None if layer.mlp is None else {"kind": "dense", "ff": layer.mlp["ff"], "limit": layer.mlp["limit"]}
+            out.append({"type": layer.kind, "mixer": {"left": l, "right": r, "left_scale": layer.left_scale,
+                                                      "right_scale": layer.right_scale}, "mlp": mlp})
+        d = {"architecture": self.architecture_name, "vocab": self.vocab_size, "width": self.hidden_size,
+             "norm": {"eps": self.norm_eps}, "layers": out}
+        if self.eos_token_id is not None:
+            d["eos_token_id"] = self.eos_token_id
+        if self.max_position_embeddings is not None:
+            d["max_position_embeddings"] = self.max_position_embeddings
+        return d
+
+    def flat(self) -> dict[str, Any]:
+        return {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "num_hidden_layers": len(self.layers),
+                "layer_kinds": [layer.kind for layer in self.layers]}

@@ -5,7 +5,9 @@
 // Formulas as in the reference's pure-torch paged path (layers/attention.py:21-40): key j of
 // the request is kept iff j <= position of the query (and j < context length); scores are
 // scale * q.k; softmax over kept keys; output = sum p_j v_j. A window w additionally keeps
-// only j > position - w (not in the reference).
+// only j > position - w (not in the reference). Three further options: `keep_first` n keeps the keys j < n visible
+// behind a window; `softcap` c > 0 bends every score to c * tanh(score / c) before the softmax; `sinks` (one float per
+// query head) adds exp(sink) to the softmax's denominator, a term without key or value.
 //
 // Keys are processed in chunks whose boundaries are multiples of the chunk size counted from
 // position 0 of the request, so the order of every sum for a given token is the same however
@@ -21,7 +23,7 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
                    const int32_t* __restrict__ block_tables, int bt_stride,
                    const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                    const int32_t* __restrict__ context_lens, int Hq, int Hkv, int D, int page, float scale,
-                   int window) {
+                   int window, int keep_first, float softcap, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   float* qs = lds;                 // D
   float* sc = lds + D;             // AS_THREADS scores / probabilities
@@ -43,14 +45,18 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
   const int hi = min(pos + 1, context_lens[b]);
   // window > 0: the last `window` keys; window < 0: a block mask, only the keys of the query's own block of -window positions
   const int lo = window > 0 ? max(0, pos - window + 1) : (window < 0 ? pos - pos % (-window) : 0);
+  // behind a window the first keep_first keys stay visible: the chunks walk [0, kept) and then [lo, hi)
+  const int kept = (window > 0 && keep_first > 0) ? min(min(keep_first, lo), hi) : 0;
   float m = -INFINITY, l = 0.f;
   // thread d < D owns output channel d (two channels per thread when D > AS_THREADS)
   float acc0 = 0.f, acc1 = 0.f;
 
-  for (int c0 = (lo / AS_THREADS) * AS_THREADS; c0 < hi; c0 += AS_THREADS) {
+  const int first_c0 = (lo / AS_THREADS) * AS_THREADS;
+  for (int c0 = kept > 0 ? 0 : first_c0; c0 < hi; c0 += AS_THREADS) {
+    if (c0 >= kept && c0 < first_c0) { c0 = first_c0 - AS_THREADS; continue; }   // nothing visible between the kept keys and the window
     const int j = c0 + tid;
     float s = -INFINITY;
-    bool keep = j >= lo && j < hi;
+    bool keep = (j >= lo || j < kept) && j < hi;
     if (keep) {
       const int64_t pg = bt[j / page];
       keep = pg >= 0;                        // a page that is not held is never dereferenced
@@ -60,6 +66,7 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
         float dot = 0.f;
         for (int d = 0; d < D; ++d) dot += qs[d] * to_f32<T>(kr[d]);
         s = dot * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       }
     }
     // chunk max
@@ -83,12 +90,13 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
     m = m_new;
     acc0 *= alpha;
     acc1 *= alpha;
-    const int jb = max(c0, lo), je = min(c0 + AS_THREADS, hi);
+    const int jb = kept > 0 ? c0 : max(c0, lo), je = min(c0 + AS_THREADS, hi);
     for (int dd = 0; dd < 2; ++dd) {
       const int d = tid + dd * AS_THREADS;
       if (d < D) {
         float a = 0.f;
         for (int jj = jb; jj < je; ++jj) {
+          if (jj < lo && jj >= kept) continue;   // its probability is 0 and its page may have been given back
           const int64_t pg = bt[jj / page];
           if (pg < 0) continue;                // its probability is 0
           const int off = jj % page;
@@ -99,6 +107,15 @@ attn_simple_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ ou
     }
     __syncthreads();
   }
+  if (sinks != nullptr) {
+    // the sink joins the denominator under the same running maximum; alone (no visible key) it leaves an output of zero
+    const float sk = sinks[h];
+    const float m_new = fmaxf(m, sk);
+    const float alpha = (m == -INFINITY) ? 0.f : expf(m - m_new);
+    l = l * alpha + expf(sk - m_new);
+    acc0 *= alpha;
+    acc1 *= alpha;
+  }
   const float inv = l > 0.f ? 1.f / l : 0.f;
   if (tid < D) out[t * out_stride + (int64_t)h * D + tid] = from_f32<T>(acc0 * inv);
   if (tid + AS_THREADS < D) out[t * out_stride + (int64_t)h * D + tid + AS_THREADS] = from_f32<T>(acc1 * inv);
@@ -108,21 +125,22 @@ extern "C" int me_attn_simple(const void* q, int64_t q_stride, void* out, int64_
                               const void* k_cache, const void* v_cache, const int32_t* block_tables,
                               int bt_stride, const int32_t* seq_of_token, const int32_t* positions,
                               const int32_t* context_lens, int64_t num_tokens, int Hq, int Hkv, int D, int page, float scale, int window,
-                              hipStream_t stream) {
+                              int keep_first, float softcap, const float* sinks, hipStream_t stream) {
   if (num_tokens == 0) return 0;
   ME_CHECK(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   ME_CHECK(D >= 1 && D <= 2 * AS_THREADS, "attention (float32 path): head_dim %d outside 1..%d", D, 2 * AS_THREADS);
   ME_CHECK(page >= 1, "attention: bad page size");
+  ME_CHECK(keep_first >= 0 && softcap >= 0.f, "attention: keep_first and softcap must not be negative");
   dim3 grid(num_tokens, Hq), block(AS_THREADS);
   size_t lds = (size_t)(D + AS_THREADS) * sizeof(float);
   if (dtype == ME_F32)
     attn_simple_kernel<float><<<grid, block, lds, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_cache, (const float*)v_cache,
-        block_tables, bt_stride, seq_of_token, positions, context_lens, Hq, Hkv, D, page, scale, window);
+        block_tables, bt_stride, seq_of_token, positions, context_lens, Hq, Hkv, D, page, scale, window, keep_first, softcap, sinks);
   else if (dtype == ME_BF16)
     attn_simple_kernel<bf16_t><<<grid, block, lds, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache,
-        block_tables, bt_stride, seq_of_token, positions, context_lens, Hq, Hkv, D, page, scale, window);
+        block_tables, bt_stride, seq_of_token, positions, context_lens, Hq, Hkv, D, page, scale, window, keep_first, softcap, sinks);
   else
     ME_CHECK(false, "attention: bad dtype code %d", dtype);
   ME_LAUNCH_CHECK();

@@ -153,6 +153,7 @@ __global__ void activation_kernel(const TX* __restrict__ x, int64_t x_stride, TX
     const float v = to_f32<TX>(x[t * x_stride + (i - t * n)]);
     float r;
     if (KIND == 0) r = silu_f(v);
+    else if (KIND == 2) r = tanhf(v);
     else { const float p = fmaxf(v, 0.f); r = p * p; }
     out[i] = from_f32<TX>(r);
   }
@@ -160,12 +161,12 @@ __global__ void activation_kernel(const TX* __restrict__ x, int64_t x_stride, TX
 
 extern "C" int me_activation(const void* x, int64_t x_stride, void* out, int dtype, int kind, int64_t T, int n, hipStream_t stream) {
   if (T == 0 || n == 0) return 0;
-  ME_CHECK(kind == 0 || kind == 1, "activation: unknown kind %d", kind);
+  ME_CHECK(kind >= 0 && kind <= 2, "activation: unknown kind %d", kind);
   const int64_t total = T * n;
   const dim3 grid((unsigned)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535)), block(256);
 #define ACT(TX, K) activation_kernel<TX, K><<<grid, block, 0, stream>>>((const TX*)x, x_stride, (TX*)out, T, n)
-  if (dtype == ME_F32) { if (kind == 0) ACT(float, 0); else ACT(float, 1); }
-  else { if (kind == 0) ACT(bf16_t, 0); else ACT(bf16_t, 1); }
+  if (dtype == ME_F32) { if (kind == 0) ACT(float, 0); else if (kind == 1) ACT(float, 1); else ACT(float, 2); }
+  else { if (kind == 0) ACT(bf16_t, 0); else if (kind == 1) ACT(bf16_t, 1); else ACT(bf16_t, 2); }
 #undef ACT
   ME_LAUNCH_CHECK();
   return 0;
@@ -223,7 +224,7 @@ __global__ void causal_conv_kernel(const TX* __restrict__ x, int64_t x_stride, c
     const int src = l0 - (taps - 1) + j;
     seen[j] = src >= 0 ? to_f32<TX>(x[(first + src) * x_stride + c]) : held[src + taps - 1];
   }
-  const float bc = bias[c];
+  const float bc = bias != nullptr ? bias[c] : 0.f;
   for (int l = l0; l < l1; ++l) {
     const float now = to_f32<TX>(x[(first + l) * x_stride + c]);
     float acc = bc + wv[taps - 1] * now;
@@ -266,7 +267,7 @@ __global__ void causal_conv_step_kernel(const TX* __restrict__ x, int64_t x_stri
   const float now = to_f32<TX>(x[(int64_t)b * x_stride + c]);
   float seen[CONV_MAX_TAPS];
   for (int s = 0; s < taps - 1; ++s) seen[s] = held[s];
-  float acc = bias[c] + w[(int64_t)c * taps + taps - 1] * now;
+  float acc = (bias != nullptr ? bias[c] : 0.f) + w[(int64_t)c * taps + taps - 1] * now;
   for (int s = 0; s < taps - 1; ++s) acc += w[(int64_t)c * taps + s] * seen[s];
   out[(int64_t)b * C + c] = from_f32<TX>(silu_f(acc));
   for (int s = 0; s + 1 < taps - 1; ++s) held[s] = seen[s + 1];
@@ -691,6 +692,7 @@ extern "C" int me_linear_recurrence(const void* q, int64_t q_stride, const void*
 
 // ------------------------------------------------------------------ unit rms per group, with a gate
 // KIND 0: u = y * silu(gate); out = u / rms_group(u) * w.    KIND 1: out = y / rms_group(y) * w * sigmoid(gate).
+// KIND 2: out = y / rms_group(y) * w * silu(gate).
 // y: `parts` stacked float32 slices [parts, T, n], added here. One workgroup per row.
 template <typename TX, int KIND>
 __global__ void gated_rms_norm_kernel(const float* __restrict__ y, int parts, int64_t part_stride, const TX* __restrict__ gate,
@@ -716,6 +718,7 @@ __global__ void gated_rms_norm_kernel(const float* __restrict__ y, int parts, in
       const int j = g * per + i;
       float r = row[j] * inv * w[j];
       if (KIND == 1) r *= sigmoid_f(to_f32<TX>(gate[t * gate_stride + j]));
+      if (KIND == 2) r *= silu_f(to_f32<TX>(gate[t * gate_stride + j]));
       out[t * n + j] = from_f32<TX>(r);
     }
   }
@@ -726,12 +729,12 @@ extern "C" int me_gated_rms_norm(const float* y, int parts, int64_t part_stride,
                                  hipStream_t stream) {
   if (T == 0) return 0;
   ME_CHECK(n >= 1 && n <= 15360 && groups >= 1 && n % groups == 0, "gated_rms_norm: width %d, %d groups", n, groups);
-  ME_CHECK(parts >= 1 && parts <= 64 && (kind == 0 || kind == 1), "gated_rms_norm: bad slice count or kind");
+  ME_CHECK(parts >= 1 && parts <= 64 && kind >= 0 && kind <= 2, "gated_rms_norm: bad slice count or kind");
   const dim3 grid((unsigned)T), block(n >= 1024 ? 256 : (n > 256 ? 128 : 64));
   const size_t lds = (size_t)n * sizeof(float);
 #define GN(TX, K) gated_rms_norm_kernel<TX, K><<<grid, block, lds, stream>>>(y, parts, part_stride, (const TX*)gate, gate_stride, w, (TX*)out, n, groups, eps)
-  if (dtype == ME_F32) { if (kind == 0) GN(float, 0); else GN(float, 1); }
-  else { if (kind == 0) GN(bf16_t, 0); else GN(bf16_t, 1); }
+  if (dtype == ME_F32) { if (kind == 0) GN(float, 0); else if (kind == 1) GN(float, 1); else GN(float, 2); }
+  else { if (kind == 0) GN(bf16_t, 0); else if (kind == 1) GN(bf16_t, 1); else GN(bf16_t, 2); }
 #undef GN
   ME_LAUNCH_CHECK();
   return 0;

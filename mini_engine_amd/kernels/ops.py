@@ -19,8 +19,9 @@ import torch
 from . import build
 
 ME_BF16, ME_F32 = 0, 1
-ACTIVATIONS = {"silu": 0, "relu2": 1}          # elementwise activations of `activation`
-GATED_NORMS = {"silu_before": 0, "sigmoid_behind": 1}
+ACTIVATIONS = {"silu": 0, "relu2": 1, "tanh": 2}          # elementwise activations of `activation`
+GATED_NORMS = {"silu_before": 0, "sigmoid_behind": 1, "silu_behind": 2}
+DECAY_RULES = {"bonus": 0, "delta": 1}         # update rules of `decay_rows_recurrence`
 _DT = {torch.bfloat16: ME_BF16, torch.float32: ME_F32}
 
 
@@ -63,7 +64,7 @@ _CORE_PROTOS = {
     "me_silu_and_mul": [P, P, I, L, I, P],
     "me_qk_norm_rope_store": [P, I, L, L, P, P, F, P, L, L, P, P, P, P, I, I, I, I, I, P],
     "me_store_kv": [P, P, I, L, L, L, P, P, P, I, I, I, P],
-    "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, P],
+    "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, I, F, P, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
@@ -85,6 +86,12 @@ _CORE_PROTOS = {
     "me_moe_gate_up": [P, L, P, P, P, P, P, P, L, I, I, I, I, I, P],
     "me_moe_down": [P, P, P, P, P, P, P, P, L, I, I, I, I, I, P],
     "me_moe_experts_simple": [P, L, I, P, P, P, P, P, P, L, I, I, I, I, P],
+    "me_add_bias": [P, I, I, L, L, P, I, P, I, L, I, P],
+    "me_sigmoid_gate": [P, L, P, L, I, L, I, P],
+    "me_glu_clamped": [P, L, P, I, L, I, F, F, P],
+    "me_weighted_sum": [I, P, P, P, P, P, P, P, P, F, P, P, P, I, L, I, P],
+    "me_token_shift": [P, L, I, P, I, P, L, P, P, P, P, L, I, P],
+    "me_decay_rows_recurrence": [P, L, P, L, P, L, P, L, P, L, I, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
     "me_sample_static": [P, L, P, P, P, I, I, P],
 }
@@ -340,10 +347,13 @@ class HipBackend:
                         positions, prefill_cu, num_decodes: int, max_decode_context: int, scale: float,
                         window: int | None, Hq: int, Hkv: int, D: int, force_simple: bool = False,
                         max_prefill_context: int = 0, even_contexts: bool = False, decode_as_prefill: bool = False,
-                        chunk: int | None = None):
+                        chunk: int | None = None, keep_first: int = 0, softcap: float | None = None, sinks=None):
         """Causal attention of this step's tokens over the paged keys of their requests. `chunk`: a block mask in
         place of a window: the query at position i sees the keys j <= i of its own block, floor(j / chunk) =
-        floor(i / chunk) (the kernels take it as a negative window).
+        floor(i / chunk) (the kernels take it as a negative window). `keep_first`: behind a window the keys j <
+        keep_first stay visible. `softcap` c: every score becomes c * tanh(score / c) before the softmax. `sinks`
+        (float32 [Hq]): exp(sink_h) joins the softmax's denominator of head h, a term without key or value. With any
+        of the three the rows take the exact kernel (`attn_simple`), whatever their dtype.
 
         q: [T, Hq*D] (a strided view is fine). Rows are ordered decode requests first (one token
         each, `num_decodes` of them), then the others; `prefill_cu` int32 [B - num_decodes + 1]
@@ -370,13 +380,17 @@ class HipBackend:
         _check(not (window and chunk), "attention: a window and a block mask exclude each other")
         win = -int(chunk) if chunk else int(window or 0)
         span = abs(win)          # no query sees more keys than this (0: all of them)
+        _check(not keep_first or (window and keep_first > 0), "attention: keys are kept behind a window only")
+        _check(sinks is None or (sinks.dtype == torch.float32 and sinks.shape == (Hq,) and sinks.is_contiguous()),
+               "attention: sinks must be float32 [Hq]")
+        plain_scores = not keep_first and not softcap and sinks is None
         mfma = (q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 512 and page >= 8 and page & (page - 1) == 0
-                and not force_simple)
+                and not force_simple and plain_scores)
         if not mfma:
             core().call("me_attn_simple", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), _code(q.dtype),
                         k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
                         seq_of_token.data_ptr(), positions.data_ptr(), context_lens.data_ptr(), T, Hq, Hkv, D, page,
-                        float(scale), win, _stream())
+                        float(scale), win, int(keep_first or 0), float(softcap or 0.0), _ptr(sinks), _stream())
             return out
         lib = attn_lib(D)
         es = q.element_size()
@@ -624,7 +638,7 @@ class HipBackend:
         return rounded, new
 
     def activation(self, x: torch.Tensor, kind: str) -> torch.Tensor:
-        """silu(x) or relu(x)^2 of a row view [T, n] (unit inner stride), float32 inside; contiguous result."""
+        """silu(x), relu(x)^2 or tanh(x) of a row view [T, n] (unit inner stride), float32 inside; contiguous result."""
         _check(x.dim() == 2 and x.stride(1) == 1 and kind in ACTIVATIONS, "activation: rows with unit inner stride, a known kind")
         T, n = x.shape
         out = torch.empty((T, n), dtype=x.dtype, device=x.device)
@@ -640,7 +654,7 @@ class HipBackend:
 
     # -- mixers with a state of fixed size -------------------------------------------------
     def causal_conv(self, x, weight, bias, state, state_slots, cu_seqlens, q_lens) -> torch.Tensor:
-        """silu(bias + sum_j weight[:, j] * x[t - (taps - 1) + j]) per channel over every request's tokens of this step,
+        """silu(bias + sum_j weight[:, j] * x[t - (taps - 1) + j]) per channel (bias None: none) over every request's tokens of this step,
         continued from its state: x a row view [T, C]; weight float32 [C, taps] (the last tap is the current
         token's); state a float32 view [slots, C * (taps - 1)] (per channel the inputs before the request's next
         token, oldest first), rows `state_slots`; it moves on by this step's tokens. `q_lens`: the requests' token
@@ -649,13 +663,13 @@ class HipBackend:
         taps = weight.shape[1]
         B = state_slots.numel()
         _check(x.stride(1) == 1 and weight.dtype == torch.float32 and weight.shape == (C, taps) and weight.is_contiguous()
-               and bias.dtype == torch.float32 and bias.shape == (C,) and bias.is_contiguous(), "causal_conv: bad operands")
+               and (bias is None or (bias.dtype == torch.float32 and bias.shape == (C,) and bias.is_contiguous())), "causal_conv: bad operands")
         _check(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] == C * (taps - 1),
                "causal_conv: state must be float32 [slots, C * (taps - 1)]")
         _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and len(q_lens) == B and sum(q_lens) == T,
                "causal_conv: metadata must be int32, one token count per request")
         out = torch.empty((T, C), dtype=x.dtype, device=x.device)
-        core().call("me_causal_conv", x.data_ptr(), x.stride(0), _code(x.dtype), weight.data_ptr(), bias.data_ptr(),
+        core().call("me_causal_conv", x.data_ptr(), x.stride(0), _code(x.dtype), weight.data_ptr(), _ptr(bias),
                     state.data_ptr(), state.stride(0), state_slots.data_ptr(), cu_seqlens.data_ptr(), max(q_lens),
                     out.data_ptr(), T, B, C, taps, _stream())
         return out
@@ -705,7 +719,8 @@ class HipBackend:
 
     def gated_rms_norm(self, y, gate, weight, eps: float, groups: int, kind: str, out_dtype: torch.dtype) -> torch.Tensor:
         """`kind` "silu_before": u = y * silu(gate), out = u / rms(u) * weight with the root mean square taken over
-        each of `groups` equal parts of a row; "sigmoid_behind": out = y / rms(y) * weight * sigmoid(gate). y float32
+        each of `groups` equal parts of a row; "sigmoid_behind": out = y / rms(y) * weight * sigmoid(gate); "silu_behind": the
+        same with silu(gate). y float32
         [T, n] or slices [S, T, n] that are added first; gate a row view [T, n] of out_dtype. Returns [T, n]."""
         if y.dim() == 3 and y.shape[0] > 64:          # more slices than the kernel adds (a state of thousands of rows)
             y = y.sum(0)
@@ -794,6 +809,116 @@ class HipBackend:
                     q.data_ptr(), q.stride(0), _code(k_cache.dtype), T, Hq, Hkv, D, page, int(vdim), int(mix),
                     _ptr(lam) if mix == 2 else None, _ptr(v_first) if mix else None, v_first.stride(0) if mix else 0, _stream())
         return q
+
+    # -- two mixers side by side: a recurrence with a decay per state row, and the steps around it -----------
+    def add_bias(self, x, bias, out_dtype: torch.dtype) -> torch.Tensor:
+        """(x summed over its slices) + bias, rounded once to out_dtype. x: a row view [T, n] or float32 partial sums
+        [P, T, n]; bias: float32 [nb], nb <= n (columns beyond nb get none). Returns contiguous [T, n]."""
+        parts = x.shape[0] if x.dim() == 3 else 1
+        T, n = x.shape[-2], x.shape[-1]
+        _check(x.stride(-1) == 1 and (x.dim() == 2 or (x.dtype == torch.float32 and x.is_contiguous())), "add_bias: rows or float32 partial sums")
+        _check(bias.dtype == torch.float32 and bias.dim() == 1 and bias.numel() <= n and bias.is_contiguous(), "add_bias: bias float32 [<= n]")
+        out = torch.empty((T, n), dtype=out_dtype, device=x.device)
+        core().call("me_add_bias", x.data_ptr(), _code(x.dtype), parts, T * n if x.dim() == 3 else 0, x.stride(-2), bias.data_ptr(),
+                    bias.numel(), out.data_ptr(), _code(out_dtype), T, n, _stream())
+        return out
+
+    def sigmoid_gate_(self, o: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+        """o *= sigmoid(gate), element by element, in place; row views [T, n] of one dtype."""
+        T, n = o.shape
+        _check(o.dim() == 2 and gate.shape == (T, n) and o.stride(1) == 1 and gate.stride(1) == 1 and gate.dtype == o.dtype,
+               "sigmoid_gate: two row views [T, n] of one dtype")
+        core().call("me_sigmoid_gate", o.data_ptr(), o.stride(0), gate.data_ptr(), gate.stride(0), _code(o.dtype), T, n, _stream())
+        return o
+
+    def glu_clamped(self, gu: torch.Tensor, limit: float, alpha: float) -> torch.Tensor:
+        """g = min(gu[:, :I], limit), u = clamp(gu[:, I:], -limit, limit); g * sigmoid(alpha * g) * (u + 1): [T, I]."""
+        _check(gu.dim() == 2 and gu.stride(1) == 1 and gu.shape[1] % 2 == 0, "glu_clamped: rows [T, 2 I]")
+        T, inter = gu.shape[0], gu.shape[1] // 2
+        out = torch.empty((T, inter), dtype=gu.dtype, device=gu.device)
+        core().call("me_glu_clamped", gu.data_ptr(), gu.stride(0), out.data_ptr(), _code(gu.dtype), T, inter, float(limit), float(alpha), _stream())
+        return out
+
+    def weighted_sum(self, terms, norm_weight=None, eps: float = 0.0, stream=None, out_dtype: torch.dtype | None = None):
+        """sum_i scale_i * (term_i + bias_i) in float32. terms: up to four (rows [T, n] in the compute dtype or float32
+        partial sums [P, T, n], a number, float32 bias [n] or None). Without `norm_weight`: returns the sum, float32
+        [T, n]. With it (float32 [n]) and `stream` (float32 [T, n]): the norm on the sum and the residual sum in the same
+        pass, stream' = stream + norm_weight * s / sqrt(mean(s^2) + eps); returns (stream' rounded to out_dtype, stream')."""
+        k = len(terms)
+        _check(1 <= k <= 4, "weighted_sum: one to four terms")
+        T, n = terms[0][0].shape[-2:]
+        ptrs, dts, parts, strides, scales, biases = (c_void_p * 4)(), (c_int * 4)(), (c_int * 4)(), (c_int64 * 4)(), (c_float * 4)(), (c_void_p * 4)()
+        for i, (t, sc, b) in enumerate(terms):
+            _check(t.is_contiguous() and t.shape[-2:] == (T, n) and (t.dim() == 2 or (t.dim() == 3 and t.dtype == torch.float32)),
+                   "weighted_sum: a term is rows [T, n] or float32 partial sums [P, T, n]")
+            _check(b is None or (b.dtype == torch.float32 and b.shape == (n,) and b.is_contiguous()), "weighted_sum: biases float32 [n]")
+            ptrs[i], dts[i], parts[i], strides[i] = t.data_ptr(), _code(t.dtype), (t.shape[0] if t.dim() == 3 else 1), T * n
+            scales[i], biases[i] = float(sc), None if b is None else b.data_ptr()
+        dev = terms[0][0].device
+        if norm_weight is None:
+            out = torch.empty((T, n), dtype=torch.float32, device=dev)
+            core().call("me_weighted_sum", k, ptrs, dts, parts, strides, scales, biases, out.data_ptr(), None, 0.0, None, None, None, 0, T, n, _stream())
+            return out
+        _check(norm_weight.dtype == torch.float32 and norm_weight.shape == (n,) and norm_weight.is_contiguous()
+               and stream is not None and stream.dtype == torch.float32 and stream.shape == (T, n) and stream.is_contiguous(),
+               "weighted_sum: norm weight float32 [n], stream float32 [T, n]")
+        new = torch.empty_like(stream)
+        rounded = new if out_dtype in (None, torch.float32) else torch.empty((T, n), dtype=out_dtype, device=dev)
+        core().call("me_weighted_sum", k, ptrs, dts, parts, strides, scales, biases, None, norm_weight.data_ptr(), float(eps),
+                    stream.data_ptr(), new.data_ptr(), None if rounded is new else rounded.data_ptr(),
+                    _code(rounded.dtype), T, n, _stream())
+        return rounded, new
+
+    def token_shift(self, x, mu, state, state_slots, cu_seqlens, seq_of_token) -> torch.Tensor:
+        """out[s, t] = x[t] + (x[t - 1] - x[t]) * mu[s] for every mix s, where x[t - 1] is the row of the request's previous
+        token: for the first of a request's tokens in this step, what its state row holds (the step function has zeroed
+        it for a request that starts at position 0); the state row then takes the request's last row of this step.
+        x: a row view [T, n]; mu: float32 [S, n]; state: a float32 view [slots, n], rows `state_slots`. Returns [S, T, n]
+        in x's dtype."""
+        T, n = x.shape
+        S = mu.shape[0]
+        B = state_slots.numel()
+        _check(x.stride(1) == 1 and mu.dtype == torch.float32 and mu.shape == (S, n) and mu.is_contiguous(), "token_shift: rows [T, n], mu float32 [S, n]")
+        _check(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == n and state.stride(1) == 1, "token_shift: state float32 [slots, n]")
+        _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and _is_i32(seq_of_token, T), "token_shift: metadata must be int32")
+        out = torch.empty((S, T, n), dtype=x.dtype, device=x.device)
+        core().call("me_token_shift", x.data_ptr(), x.stride(0), _code(x.dtype), mu.data_ptr(), S, state.data_ptr(), state.stride(0),
+                    state_slots.data_ptr(), cu_seqlens.data_ptr(), seq_of_token.data_ptr(), out.data_ptr(), T, n, _stream())
+        return out
+
+    def decay_rows_recurrence(self, q, k, v, raw, state, state_slots, cu_seqlens, q_lens, H: int, G: int, N: int, P: int, rule: str,
+                              base, rate=None, bonus=None, beta=None, unit_eps: float | None = None, q_scale: float = 1.0) -> torch.Tensor:
+        """Per request and head a float32 state S [N, P] whose rows decay each at a rate the token chooses, walked over
+        the request's tokens of this step in order from its state row, which is left at the state behind the last token.
+        rule "bonus":  d = exp(-exp(raw + base));  y = (S + diag(bonus) k v^T)^T q;  S <- diag(d) S + k v^T.
+        rule "delta":  d = exp(-rate_h softplus(raw + base));  S <- diag(d) S;  u = sigmoid(beta) (v - S^T k);
+                       S <- S + k u^T;  y = S^T q.
+        q, k: row views [T, G * N] (heads share them by groups of H / G); v: [T, H * P]; raw: [T, H * N]; beta: [T, H];
+        base, bonus: float32 [H * N]; rate: float32 [H]. `unit_eps`: q and k are made unit vectors per head first, x /
+        sqrt(sum(x^2) + unit_eps); q is multiplied by q_scale. Everything but the rows read is float32. Returns float32
+        [T, H * P]. (`q_lens`: the requests' token counts on the host.)"""
+        T, B = v.shape[0], state_slots.numel()
+        dtype = v.dtype
+        _check(rule in DECAY_RULES, f"decay_rows_recurrence: rule must be one of {sorted(DECAY_RULES)}")
+        for t, width in ((q, G * N), (k, G * N), (v, H * P), (raw, H * N)):
+            _check(t.dim() == 2 and t.shape == (T, width) and t.stride(1) == 1 and t.dtype == dtype, "decay_rows_recurrence: bad q, k, v or decay rows")
+        _check(state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1 and state.shape[1] == H * N * P,
+               "decay_rows_recurrence: state must be float32 [slots, H * N * P]")
+        for w, width in ((base, H * N), (bonus, H * N), (rate, H)):
+            _check(w is None or (w.dtype == torch.float32 and w.numel() == width and w.is_contiguous()), "decay_rows_recurrence: constants float32")
+        _check(base is not None and (bonus is not None if rule == "bonus" else (rate is not None and beta is not None)),
+               "decay_rows_recurrence: the rule's constants are missing")
+        if beta is not None:
+            _check(beta.shape == (T, H) and beta.stride(1) == 1 and beta.dtype == dtype, "decay_rows_recurrence: write strengths [T, H]")
+        _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and len(q_lens) == B and sum(q_lens) == T, "decay_rows_recurrence: metadata")
+        _check(1 <= N <= 256 and H % G == 0, "decay_rows_recurrence: up to 256 state rows, heads a multiple of the groups")
+        y = torch.empty((T, H * P), dtype=torch.float32, device=v.device)
+        core().call("me_decay_rows_recurrence", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
+                    raw.data_ptr(), raw.stride(0), _ptr(beta), 0 if beta is None else beta.stride(0), _code(dtype),
+                    base.data_ptr(), _ptr(rate), _ptr(bonus), state.data_ptr(), state.stride(0), state_slots.data_ptr(),
+                    cu_seqlens.data_ptr(), y.data_ptr(), B, H, G, N, P, DECAY_RULES[rule], int(unit_eps is not None),
+                    float(unit_eps or 0.0), float(q_scale), decay_row_groups(B, H, N, P), _stream())
+        return y
 
     # -- routed experts ------------------------------------------------------------------
     def moe_route(self, x, router, top: int, group_count: int = 1, group_keep: int = 1):
@@ -1360,6 +1485,15 @@ def expert_tile_rows(T: int, top: int, E: int) -> int:
     return 128 if T * top >= EXPERT_LARGE_TILE_ROWS * E else 64
 
 
+def decay_row_groups(num_seqs: int, H: int, N: int, P: int) -> int:
+    """Lanes that share a column of the state in `decay_rows_recurrence`: 4 (a quarter of the rows per lane, four times the
+    waves) where a lane could not keep a whole column in registers, or while one lane to a column leaves compute units
+    without a wave; else 1 (no exchange between lanes)."""
+    if N > 64:
+        return 4
+    return 4 if num_seqs * H * -(-P // 64) < 2 * _COMPUTE_UNITS and N >= 16 else 1
+
+
 def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:
     """Whether `rows` rows against the packed gate/up weight w [2 I, K] are few enough, and w of a kind, for the
     gating to happen in the product's epilogue: a bfloat16 product that the unsplit skinny kernel takes, up to
@@ -1466,6 +1600,12 @@ def gated_rms_norm(*a, **k): return backend().gated_rms_norm(*a, **k)
 def scaled_sum_norm(*a, **k): return backend().scaled_sum_norm(*a, **k)
 def softcap_(*a, **k): return backend().softcap_(*a, **k)
 def qkv_prepare_store(*a, **k): return backend().qkv_prepare_store(*a, **k)
+def add_bias(*a, **k): return backend().add_bias(*a, **k)
+def sigmoid_gate_(*a, **k): return backend().sigmoid_gate_(*a, **k)
+def glu_clamped(*a, **k): return backend().glu_clamped(*a, **k)
+def weighted_sum(*a, **k): return backend().weighted_sum(*a, **k)
+def token_shift(*a, **k): return backend().token_shift(*a, **k)
+def decay_rows_recurrence(*a, **k): return backend().decay_rows_recurrence(*a, **k)
 def moe_route(*a, **k): return backend().moe_route(*a, **k)
 def routed_experts(*a, **k): return backend().routed_experts(*a, **k)
 def route_and_run_experts(*a, **k): return backend().route_and_run_experts(*a, **k)

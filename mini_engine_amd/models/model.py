@@ -69,7 +69,10 @@ class DecoderModel(Part):
         for call in self.order:
             layer = self.layers[call.layer]
             if call.cache_of is not None and hasattr(layer, "cache_need") and layer.cache_need() is not None:
-                readers.setdefault(call.cache_of, []).append(layer.cache_need().own_rule())
+                theirs = layer.cache_need()
+                readers.setdefault(call.cache_of, []).append(theirs.own_rule())
+                if theirs.keep_first:
+                    readers[call.cache_of].append(("first", int(theirs.keep_first)))
         for i, call in enumerate(self.order):
             layer = self.layers[call.layer]
             need: CacheNeed | None = layer.cache_need() if hasattr(layer, "cache_need") else None

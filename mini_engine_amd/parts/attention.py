@@ -44,6 +44,14 @@ class Attention(Mixer):
     and `value_mix`: "first" keeps this layer's values of the step's tokens under `value_mix_key` in the step's shared
     values; "blend" replaces its own by (1 - lambda) v + lambda v_first with a learned scalar lambda (`vmix`) before
     they are cached. Layers that share a key have the same number of value dimensions.
+
+    Options of the mask and the softmax (they go to the attention kernels as they are): `keep_first` (behind the window
+    the keys at positions below it stay visible, at their true positions), `score_cap` c (a score s becomes c * tanh(s /
+    c)), `sinks` (a learned number per query head whose exponential joins the softmax's denominator without a key or a
+    value). Options around the products: `output_gate` (the concatenated heads are multiplied element by element by the
+    sigmoid of further output features of the packed product, as many as the heads' values), `out_bias` (a bias on the
+    output product), and `qkv_bias` together with per-head norms or a position encoding (the biases are then added to
+    the packed product's unrounded sums by a kernel of their own in front of the per-head norm and rotation).
     """
 
     takes_pending_norm = True      # x goes to the packed product and nowhere else
@@ -52,7 +60,9 @@ class Attention(Mixer):
                  scale: float, qk_norm_eps: float | None = None, position: PositionEncoding | None = None,
                  window: int | None = None, own_kv: bool = True, value_dim: int | None = None,
                  chunk: int | None = None, head_gate: bool = False, qkv_bias: bool = False, qk_norm_over: str = "head",
-                 q_temperature: tuple | None = None, value_mix: str | None = None, value_mix_key: str = "v_first"):
+                 q_temperature: tuple | None = None, value_mix: str | None = None, value_mix_key: str = "v_first",
+                 keep_first: int = 0, score_cap: float | None = None, sinks: bool = False, output_gate: bool = False,
+                 out_bias: bool = False):
         super().__init__()
         if qk_norm_over not in ("head", "projection") or value_mix not in (None, "first", "blend"):
             raise ValueError("qk_norm_over is 'head' or 'projection', value_mix None, 'first' or 'blend'")
@@ -62,8 +72,16 @@ class Attention(Mixer):
         if self.q_temperature is not None and self.q_temperature[1] < 1:
             raise ValueError("the query temperature's period must be positive")
         self.value_mix, self.value_mix_key = value_mix, value_mix_key
-        self.prologue = bool(qkv_bias or qk_norm_over == "projection" or q_temperature is not None or value_mix)
-        if self.prologue and (position is not None or not own_kv or head_gate or (qk_norm_eps is not None and qk_norm_over == "head")):
+        self.keep_first, self.score_cap = int(keep_first or 0), (float(score_cap) if score_cap else None)
+        self.output_gate, self.out_bias_on = bool(output_gate), bool(out_bias)
+        if self.keep_first and not window:
+            raise ValueError("keys are kept behind a window only")
+        if head_gate and output_gate:
+            raise ValueError("a gate per head and a gate per element exclude each other")
+        per_head_path = (position is not None or not own_kv or head_gate or output_gate
+                         or (qk_norm_eps is not None and qk_norm_over == "head"))
+        self.prologue = bool(qk_norm_over == "projection" or q_temperature is not None or value_mix or (qkv_bias and not per_head_path))
+        if self.prologue and per_head_path:
             raise ValueError("biases, whole-projection norms, query temperatures and value mixing come without a position "
                              "encoding, head gates or per-head norms, on keys and values of the layer's own")
         if num_heads % num_kv_heads:
@@ -98,9 +116,11 @@ class Attention(Mixer):
             blocks.update(k=stored_k, v=stored_v)
         if head_gate:
             blocks["g"] = num_heads
+        if output_gate:
+            blocks["g"] = num_heads * self.value_dim
         self.add_child("qkv", Linear(hidden_size, sum(blocks.values()), parts=blocks))
         self.add_child("o", Linear(num_heads * self.value_dim, hidden_size))
-        rows = self.q_size + (2 * self.kv_size if own_kv else 0) + (num_heads if head_gate else 0)
+        rows = self.q_size + (2 * self.kv_size if own_kv else 0) + (num_heads if head_gate else 0) + (self.q_size if output_gate else 0)
         self._relayout = self._relayout or rows % 8 != 0
         self.gate_at = self.q_size + (2 * self.kv_size if own_kv else 0)      # first gate column of the kernels' rows
         self._laid_out = False
@@ -111,6 +131,14 @@ class Attention(Mixer):
                 self.add_param("k_norm_weight", ParamSpec((stored_k if whole else self.stored_dim,), init="norm", dtype="float32"))
         if qkv_bias:
             self.add_param("qkv_bias", ParamSpec((stored_q + stored_k + stored_v,), init="matrix", dtype="float32"))
+        if sinks:
+            self.add_param("sinks", ParamSpec((num_heads,), init="matrix", dtype="float32"))
+        else:
+            self.sinks = None
+        if out_bias:
+            self.add_param("o_bias", ParamSpec((hidden_size,), init="matrix", dtype="float32"))
+        else:
+            self.o_bias = None
         if value_mix == "blend":
             self.add_param("vmix", ParamSpec((), init=_half, dtype="float32"))
         self.norm_eps = qk_norm_eps
@@ -120,7 +148,7 @@ class Attention(Mixer):
             self.position = None
 
     def cache_need(self):
-        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window, self.chunk)
+        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window, self.chunk, self.keep_first)
 
     def set_param(self, local, tensor):
         super().set_param(local, tensor)
@@ -150,6 +178,9 @@ class Attention(Mixer):
             at += stored_k + G * nv
         if self.head_gate:
             parts.append(w[at:at + H])
+        if self.output_gate:                 # the gates take the slots of the values they multiply
+            keep_o = torch.tensor(list(range(nv)) + [-1] * (D - nv), dtype=torch.long)
+            parts.append(heads(w[at:at + H * nv], H, nv, keep_o))
         rows = sum(p.shape[0] for p in parts)
         if rows % 8:
             parts.append(w.new_zeros(8 - rows % 8, hidden))
@@ -208,8 +239,14 @@ class Attention(Mixer):
             return self._forward_with_prologue(x, step, cache)
         Hq, Hkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         grp = step.groups[cache.group]
-        packed = self.qkv.forward(x)
+        if self.qkv_bias_on:                # the bias joins the unrounded sums; one rounding behind it
+            dtype = self.qkv.weight.dtype
+            packed = ops.add_bias(self.qkv.forward(x, out_dtype=torch.float32), self.qkv_bias, dtype)
+        else:
+            packed = self.qkv.forward(x)
         gated = self.head_gate
+        extras = dict(keep_first=self.keep_first, softcap=self.score_cap, sinks=self.sinks)
+        plain_scores = not self.keep_first and self.score_cap is None and self.sinks is None
         # the kernels' rows end where the gate columns (and the padding to whole steps of 8) begin
         qkv = packed if packed.shape[1] == self.gate_at else packed[:, : self.gate_at]
         store = self.own_kv and cache.write
@@ -218,14 +255,14 @@ class Attention(Mixer):
         table = self.position.rotary_table() if self.position is not None else None
         eps = self.qk_norm_eps or 0.0
         if (store and step.num_decodes == step.num_tokens and (self.position is None or table is not None)
-                and ops.decode_step_fuses(qkv.dtype, D, cache.page_size)):
+                and plain_scores and ops.decode_step_fuses(qkv.dtype, D, cache.page_size)):
             # only single tokens: norm, rotary, cache write and attention in one launch
             o = ops.decode_step_attention(qkv, qw, kw, eps, table, cache.k, cache.v, cache.page_size, grp.block_tables,
                                           step.context_lens, step.max_decode_context, self.scale, self.window,
                                           Hq, Hkv, D, even_contexts=step.decode_contexts_even, chunk=self.chunk)
             if gated:
                 ops.head_gate(o, packed[:, self.gate_at:self.gate_at + Hq], Hq, D)
-            return self.o.forward(o, allow_partials=True)
+            return self._project(o, packed)
         if self.position is None or table is not None:
             # norm + rotary + cache write in one pass
             bound = max(step.max_decode_context, step.max_prefill_context)
@@ -253,7 +290,16 @@ class Attention(Mixer):
                                 step.seq_of_token, step.positions, step.prefill_cu, step.num_decodes,
                                 step.max_decode_context, self.scale, self.window, Hq, Hkv, D,
                                 max_prefill_context=step.max_prefill_context,
-                                even_contexts=step.decode_contexts_even, chunk=self.chunk)
+                                even_contexts=step.decode_contexts_even, chunk=self.chunk, **extras)
         if gated:
             ops.head_gate(o, packed[:, self.gate_at:self.gate_at + Hq], Hq, D)
-        return self.o.forward(o, allow_partials=True)
+        return self._project(o, packed)
+
+    def _project(self, o, packed):
+        """The element gate, the output product and its bias."""
+        if self.output_gate:
+            ops.sigmoid_gate_(o, packed[:, self.gate_at:self.gate_at + self.q_size])
+        y = self.o.forward(o, allow_partials=True)
+        if self.out_bias_on:
+            y = ops.add_bias(y, self.o_bias, self.o.weight.dtype)
+        return y

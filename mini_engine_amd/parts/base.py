@@ -63,7 +63,8 @@ class CacheNeed:
 
     ``window``: n keeps the last n positions; ``chunk``: c keeps the positions of the block of c
     positions (counted from 0) that the next token falls into; neither: every token stays. Pages that
-    the rule has passed are given back. ``readers``: the rules of other layer calls that read these
+    the rule has passed are given back. ``keep_first``: the first so many positions stay whatever the
+    rule has passed. ``readers``: the rules of other layer calls that read these
     pages (the model fills it in): the loosest of all rules holds. Layers with equal needs share one
     group of pages and one block table per request.
     """
@@ -72,14 +73,15 @@ class CacheNeed:
     window: int | None = None
     chunk: int | None = None
     readers: tuple = ()                # own_rule() of every call that reads the pages of this one
+    keep_first: int = 0
 
     @classmethod
     def keys_and_values(cls, num_kv_heads: int, head_dim: int, window: int | None = None,
-                        chunk: int | None = None) -> "CacheNeed":
+                        chunk: int | None = None, keep_first: int = 0) -> "CacheNeed":
         """The layout of the attention kernels: K [pages, heads, page, head size], V [pages, heads, head
         size, page] (V transposed inside a page: the P.V operand of the matrix cores is then one load)."""
         return cls((PageTensor("k", (num_kv_heads, PAGE, head_dim)), PageTensor("v", (num_kv_heads, head_dim, PAGE))),
-                   window, chunk)
+                   window, chunk, keep_first=int(keep_first or 0))
 
     def own_rule(self) -> tuple:
         """("window", n), ("chunk", c) or ("all", 0)."""
@@ -91,11 +93,15 @@ class CacheNeed:
 
     def keep(self):
         """What the cache manager is told: None (every token stays), an int (one trailing window), or a tuple of
-        ("window" | "chunk", n) rules of which the loosest holds at every moment."""
-        rules = {self.own_rule(), *self.readers}
+        ("window" | "chunk", n) rules of which the loosest holds at every moment, with ("first", n) among them when
+        the first n positions stay for good."""
+        rules = {self.own_rule(), *(r for r in self.readers if r[0] != "first")}
         if ("all", 0) in rules:
             return None
+        pinned = max([self.keep_first] + [r[1] for r in self.readers if r[0] == "first"])
         rules = tuple(sorted(rules))
+        if pinned > 0:
+            return rules + (("first", int(pinned)),)
         return rules[0][1] if len(rules) == 1 and rules[0][0] == "window" else rules
 
     def group_key(self) -> tuple:

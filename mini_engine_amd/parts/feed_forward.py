@@ -45,3 +45,22 @@ class ActivatedMLP(FeedForward):
 
     def forward(self, x):
         return self.down.forward(ops.activation(self.up.forward(x), self.activation), allow_partials=True)
+
+
+@register_part("feed_forward", "clamped_glu")
+class ClampedGLU(FeedForward):
+    """g = min(gate(x), limit), u = clamp(up(x), -limit, limit); down(g * sigmoid(alpha * g) * (u + 1)). Gate and up are
+    one packed product with gate's rows first."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, limit: float, alpha: float = 1.702):
+        super().__init__()
+        if not limit > 0:
+            raise ValueError("the limit must be positive")
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.limit, self.alpha = float(limit), float(alpha)
+        self.add_child("gate_up", Linear(hidden_size, 2 * intermediate_size,
+                                         parts={"gate": intermediate_size, "up": intermediate_size}))
+        self.add_child("down", Linear(intermediate_size, hidden_size))
+
+    def forward(self, x):
+        return self.down.forward(ops.glu_clamped(self.gate_up.forward(x), self.limit, self.alpha), allow_partials=True)

@@ -36,17 +36,23 @@ def architectures() -> list:
     return sorted(_BUILDERS)
 
 
-def build_model(model_config, checkpoint_names=None):
+def build_model(model_config, checkpoint_names=None, checkpoint_shapes=None):
     """Build the (unloaded) model of a typed config. A builder that has a parameter `checkpoint_names`
     is told which tensors the checkpoint stores (None: there is no checkpoint, weights will be drawn),
-    for architectures whose shape depends on it (a head that is stored or not)."""
+    for architectures whose shape depends on it (a head that is stored or not); one with a parameter
+    `checkpoint_shapes` gets their shapes by name, for sizes that only the tensors give (the inner width
+    of a product of two thin matrices)."""
     import inspect
 
     builder = builder_for(type(model_config).architecture_name)
-    if "checkpoint_names" in inspect.signature(builder).parameters:
-        return builder(model_config, checkpoint_names=checkpoint_names)
-    return builder(model_config)
+    wants = inspect.signature(builder).parameters
+    extra = {}
+    if "checkpoint_names" in wants:
+        extra["checkpoint_names"] = checkpoint_names
+    if "checkpoint_shapes" in wants:
+        extra["checkpoint_shapes"] = checkpoint_shapes
+    return builder(model_config, **extra)
 
 
 def _load_builtin() -> None:
-    from .models import negosun, qwen3, sigosun  # noqa: F401  (they register themselves)
+    from .models import negosun, qwen3, sigosun, tavevik  # noqa: F401  (they register themselves)

@@ -144,7 +144,7 @@ def load_model(model_dir: str, device, dtype: torch.dtype, max_positions: int, m
         from .random_init import fill_random
         return fill_random(build_model(cfg), random_weights, device, dtype, max_positions, on_device=True)
     index = checkpoint_index(model_dir)
-    model = build_model(cfg, checkpoint_names=set(index))
+    model = build_model(cfg, checkpoint_names=set(index), checkpoint_shapes={n: e[1] for n, e in index.items()})
     load_weights(model, model_dir, device, dtype, index)
     model.finalize_all(device, dtype, max_positions)
     return model

@@ -83,7 +83,7 @@ def store_kv(k, v, slots, k_cache, v_cache, page):
 def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_of_token, positions,
                     prefill_cu, num_decodes, max_decode_context, scale, window, Hq, Hkv, D,
                     force_simple=False, max_prefill_context=0, even_contexts=False, compute_dtype=torch.float32,
-                    chunk=None, decode_as_prefill=False):
+                    chunk=None, decode_as_prefill=False, keep_first=0, softcap=None, sinks=None):
     """Token by token: gather the keys this token may see through its request's block table
     and nothing else (so unowned pages are never read), softmax, weighted sum."""
     T = q.shape[0]
@@ -100,6 +100,8 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
             out[t] = 0
             continue
         js = torch.arange(lo, hi, device=q.device)
+        if keep_first and window and lo > 0:               # the first positions stay visible behind the window
+            js = torch.cat((torch.arange(0, min(keep_first, lo, hi), device=q.device), js))
         pages = block_tables[b, (js // page).long()].long()
         assert (pages >= 0).all(), "attention would read a page the request does not hold"
         offs = js % page
@@ -107,7 +109,13 @@ def paged_attention(q, k_cache, v_cache, page, block_tables, context_lens, seq_o
         v = v_cache[pages, :, :, offs].to(compute_dtype)             # [n, Hkv, D]
         qt = q[t].to(compute_dtype).view(Hkv, G, D)                  # query head h belongs to key head h // G
         s = torch.einsum("nkd,kgd->kgn", k, qt) * scale
-        p = torch.softmax(s, dim=-1)
+        if softcap:
+            s = softcap * torch.tanh(s / softcap)
+        if sinks is not None:                              # one more term in the denominator, no key, no value
+            s = torch.cat((s, sinks.to(compute_dtype).view(Hkv, G, 1)), dim=-1)
+            p = torch.softmax(s, dim=-1)[..., :-1]
+        else:
+            p = torch.softmax(s, dim=-1)
         out[t] = torch.einsum("kgn,nkd->kgd", p, v).reshape(Hq * D).to(q.dtype)
     return out
 
@@ -174,7 +182,7 @@ def add_rms_norm(y, weight, eps, stream, out_dtype):
 
 def activation(x, kind):
     v = x.float()
-    v = v * torch.sigmoid(v) if kind == "silu" else torch.relu(v) ** 2
+    v = v * torch.sigmoid(v) if kind == "silu" else (torch.tanh(v) if kind == "tanh" else torch.relu(v) ** 2)
     return v.to(x.dtype)
 
 
@@ -197,7 +205,7 @@ def causal_conv(x, weight, bias, state, state_slots, cu_seqlens, q_lens):
             continue
         held = state[slots[b]].view(C, taps - 1).t()                  # [taps - 1, C]
         seen = torch.cat((held, x[lo:hi].float()), 0)                  # [taps - 1 + n, C]
-        acc = bias.float().expand(hi - lo, C).clone()
+        acc = bias.float().expand(hi - lo, C).clone() if bias is not None else torch.zeros((hi - lo, C), device=x.device)
         for j in range(taps):
             acc += weight[:, j].float() * seen[j:j + hi - lo]
         out[lo:hi] = (acc * torch.sigmoid(acc)).to(x.dtype)
@@ -250,7 +258,91 @@ def gated_rms_norm(y, gate, weight, eps, groups, kind, out_dtype):
     r = (r * torch.rsqrt(r.pow(2).mean(-1, keepdim=True) + eps)).view(T, n) * weight
     if kind == "sigmoid_behind":
         r = r * torch.sigmoid(g)
+    if kind == "silu_behind":
+        r = r * (g * torch.sigmoid(g))
     return r.to(out_dtype)
+
+
+def add_bias(x, bias, out_dtype):
+    r = (x.float().sum(0) if x.dim() == 3 else x.float()).clone()
+    r[:, : bias.numel()] += bias
+    return r.to(out_dtype)
+
+
+def sigmoid_gate_(o, gate):
+    o.copy_((o.float() * torch.sigmoid(gate.float())).to(o.dtype))
+    return o
+
+
+def glu_clamped(gu, limit, alpha):
+    inter = gu.shape[1] // 2
+    g = torch.clamp(gu[:, :inter].float(), max=limit)
+    u = torch.clamp(gu[:, inter:].float(), -limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def weighted_sum(terms, norm_weight=None, eps=0.0, stream=None, out_dtype=None):
+    total = None
+    for t, sc, b in terms:
+        v = t.float().sum(0) if t.dim() == 3 else t.float()
+        if b is not None:
+            v = v + b
+        total = sc * v if total is None else total + sc * v
+    if norm_weight is None:
+        return total
+    new = stream + norm_weight * (total * torch.rsqrt(total.pow(2).mean(-1, keepdim=True) + eps))
+    return (new if out_dtype in (None, torch.float32) else new.to(out_dtype)), new
+
+
+def token_shift(x, mu, state, state_slots, cu_seqlens, seq_of_token):
+    T, n = x.shape
+    out = torch.empty((mu.shape[0], T, n), dtype=x.dtype, device=x.device)
+    cu, slots = cu_seqlens.tolist(), state_slots.tolist()
+    for b in range(len(slots)):
+        lo, hi = cu[b], cu[b + 1]
+        if hi <= lo:
+            continue
+        now = x[lo:hi].float()
+        before = torch.cat((state[slots[b]][None, :].clone(), now[:-1]), 0)
+        out[:, lo:hi] = (now[None] + (before - now)[None] * mu[:, None, :]).to(x.dtype)
+        state[slots[b]] = now[-1]
+    return out
+
+
+def decay_rows_recurrence(q, k, v, raw, state, state_slots, cu_seqlens, q_lens, H, G, N, P, rule, base, rate=None, bonus=None,
+                          beta=None, unit_eps=None, q_scale=1.0):
+    """Token by token, float32. rule "bonus": y = (S + diag(bonus) k v^T)^T q, S <- diag(d) S + k v^T with d =
+    exp(-exp(raw + base)); rule "delta": S <- diag(d) S with d = exp(-rate softplus(raw + base)), u = sigmoid(beta) (v -
+    S^T k), S <- S + k u^T, y = S^T q."""
+    T = v.shape[0]
+    y = torch.zeros((T, H * P), dtype=torch.float32, device=v.device)
+    cu, slots = cu_seqlens.tolist(), state_slots.tolist()
+    per = H // G
+    for b in range(len(slots)):
+        S = state[slots[b]].view(H, N, P).clone()
+        for t in range(cu[b], cu[b + 1]):
+            qt = q[t].float().view(G, N).repeat_interleave(per, 0)
+            kt = k[t].float().view(G, N).repeat_interleave(per, 0)
+            vt = v[t].float().view(H, P)
+            if unit_eps is not None:
+                qt = qt / torch.sqrt(qt.pow(2).sum(-1, keepdim=True) + unit_eps)
+                kt = kt / torch.sqrt(kt.pow(2).sum(-1, keepdim=True) + unit_eps)
+            qt = qt * q_scale
+            z = raw[t].float().view(H, N) + base.view(H, N)
+            if rule == "bonus":
+                d = torch.exp(-torch.exp(z))
+                kv = kt[:, :, None] * vt[:, None, :]
+                out = torch.einsum("hnp,hn->hp", S + bonus.view(H, N)[:, :, None] * kv, qt)
+                S = d[:, :, None] * S + kv
+            else:
+                d = torch.exp(-rate[:, None] * softplus(z))
+                S = d[:, :, None] * S
+                u = torch.sigmoid(beta[t].float())[:, None] * (vt - torch.einsum("hnp,hn->hp", S, kt))
+                S = S + kt[:, :, None] * u[:, None, :]
+                out = torch.einsum("hnp,hn->hp", S, qt)
+            y[t] = out.reshape(-1)
+        state[slots[b]] = S.reshape(-1)
+    return y
 
 
 def scaled_sum_norm(stream, terms, mult, w1, w2, eps, out_dtype):
@@ -417,6 +509,12 @@ class PlainBackend:
     scaled_sum_norm = staticmethod(scaled_sum_norm)
     softcap_ = staticmethod(softcap_)
     qkv_prepare_store = staticmethod(qkv_prepare_store)
+    add_bias = staticmethod(add_bias)
+    sigmoid_gate_ = staticmethod(sigmoid_gate_)
+    glu_clamped = staticmethod(glu_clamped)
+    weighted_sum = staticmethod(weighted_sum)
+    token_shift = staticmethod(token_shift)
+    decay_rows_recurrence = staticmethod(decay_rows_recurrence)
     moe_route = staticmethod(moe_route)
     routed_experts = staticmethod(routed_experts)
     route_and_run_experts = staticmethod(route_and_run_experts)
