@@ -130,8 +130,12 @@ def prefill_flops(model, T: int) -> float:
     wants logits."""
     per_token, head = _matrix_params(model)
     attn = 0.0
+    mixers = []
     for call in model.order:
         mixer = getattr(model.layers[call.layer], "mixer", None)
+        sides = [getattr(mixer, side, None) for side in ("left", "right")]        # two mixers side by side count each
+        mixers += [m for m in sides if m is not None] if any(m is not None for m in sides) else [mixer]
+    for mixer in mixers:
         heads, size = getattr(mixer, "num_heads", None), getattr(mixer, "head_dim", None)
         if heads and size:
             window, chunk = getattr(mixer, "window", None), getattr(mixer, "chunk", None)
@@ -142,7 +146,7 @@ def prefill_flops(model, T: int) -> float:
         elif heads and hasattr(mixer, "state_need"):
             # a state of N x P per head: one multiply-add to move it on and one to read it, per token
             rows = getattr(mixer, "state_dim", None) or getattr(mixer, "key_dim", 0)
-            attn += 4.0 * heads * rows * mixer.value_dim * T
+            attn += 4.0 * heads * rows * getattr(mixer, "value_dim", rows) * T
     return 2.0 * T * per_token + attn + 2.0 * head
 
 
@@ -467,7 +471,7 @@ def main(argv=None) -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="fetch every decode step's tokens before the next step is launched")
-    ap.add_argument("--design", default=None, choices=["sigosun", "negosun"],
+    ap.add_argument("--design", default=None, choices=["sigosun", "negosun", "tavevik"],
                     help="instead of the default workload: prefill and decode throughput of this design at the layer sizes "
                          "named by --design-sizes (random weights), each beside Qwen3 at the same width, depth and vocabulary")
     ap.add_argument("--design-sizes", default="0.6b,8b")

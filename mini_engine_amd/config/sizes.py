@@ -3,7 +3,7 @@ with random weights (no model folder at hand). The figures are those of the publ
 files; a model folder's own config.json always wins where there is one."""
 from __future__ import annotations
 
-from .model_config import NegosunConfig, Qwen3Config, SigosunConfig
+from .model_config import NegosunConfig, Qwen3Config, SigosunConfig, TavevikConfig
 
 SIZES = {
     # name: (layers, hidden, q heads, kv heads, head_dim, intermediate, vocab, tied)
@@ -76,12 +76,39 @@ def negosun_config(size: str, layers: int | None = None):
                                     "logit_softcap": 30.0, "layers": [layer] * n, "max_position_embeddings": 40960}), L
 
 
+def tavevik_config(size: str, layers: int | None = None):
+    """(a Tavevik configuration whose layers resemble that size's: the same width, vocabulary, feed-forward width and
+    attention heads, with `layers` layers or as many as the size has; that count). The two layer kinds take turns, the
+    second kind first. Attention under a window of 1,024 positions, half of each head's dimensions turning; in the first
+    kind 16 kept positions and a cap of 50 on the scores. Beside it a delta rule with a quarter of the attention's heads
+    at its head size (half as many key heads, four taps) or a shifted-mix recurrence with heads of 64 over the model's
+    width; thin pairs of 64."""
+    L, h, Hq, Hkv, D, I, V, _ = SIZES[size]
+    n = layers or L
+    small = D < 64
+    left = lambda first: dict({"heads": Hq, "kv_heads": Hkv, "dim": D, "vdim": D, "scale": D ** -0.5, "rot": {"dims": D // 2, "base": 1e6},
+                               "mask": dict({"size": 1024}, **({"keep_first": 16} if first else {}))}, **({"softcap": 50.0} if first else {}))
+    rank = 8 if small else 64
+    delta_heads = max(2, Hq // 4)
+    one = {"type": "parallel", "mlp": {"kind": "dense", "ff": I, "limit": 7.0},
+           "mixer": {"left": left(True), "right": {"heads": max(1, h // (16 if small else 64)), "dim": 16 if small else 64, "decay_rank": rank},
+                     "left_scale": 0.8, "right_scale": 1.1}}
+    two = {"type": "parallel_2", "mlp": {"kind": "dense", "ff": I, "limit": 7.0},
+           "mixer": {"left": left(False), "right": {"heads": delta_heads, "kv_heads": delta_heads // 2, "dim": D, "vdim": D, "conv": 4,
+                                                    "decay_rank": rank, "gate_rank": rank},
+                     "left_scale": 0.6, "right_scale": 0.9}}
+    return TavevikConfig.from_dict({"architecture": "Tavevik", "vocab": V, "width": h, "norm": {"eps": 1e-6},
+                                    "layers": [two if i % 2 == 0 else one for i in range(n)], "max_position_embeddings": 40960}), L
+
+
 def named_config(name: str, layers: int | None = None):
     """(configuration, full layer count) of a name the command lines take for random weights: a Qwen3 size
-    ("0.6b"), or "sigosun:<size>" / "negosun:<size>" for those designs at that size's layer sizes."""
+    ("0.6b"), or "sigosun:<size>" / "negosun:<size>" / "tavevik:<size>" for those designs at that size's layer sizes."""
     design, _, size = name.rpartition(":")
-    if size not in SIZES or design not in ("", "qwen3", "sigosun", "negosun"):
-        raise KeyError(f"{name!r} is not one of {sorted(SIZES)}, optionally behind 'sigosun:' or 'negosun:'")
+    if size not in SIZES or design not in ("", "qwen3", "sigosun", "negosun", "tavevik"):
+        raise KeyError(f"{name!r} is not one of {sorted(SIZES)}, optionally behind 'sigosun:', 'negosun:' or 'tavevik:'")
     if design == "negosun":
         return negosun_config(size, layers)
+    if design == "tavevik":
+        return tavevik_config(size, layers)
     return sigosun_config(size, layers) if design == "sigosun" else model_config(size, layers)

@@ -84,7 +84,34 @@ struct AttnArgs {
   const float* rope;            // [positions, HD/2, 2] (cos, sin), or nullptr: no rotation
   bf16_t* k_cache_w;
   bf16_t* v_cache_w;
+  // a score s becomes softcap * tanh(s / softcap) before the softmax (0: no cap; compiled in with ME_ATTN_SOFTCAP only)
+  float softcap;
+  // [rows, Hq] or nullptr: the natural logarithm of every (token, head)'s softmax denominator, -inf where it saw no key,
+  // for a caller that joins further terms to the softmax afterwards
+  float* lse_out;
 };
+
+#ifndef ME_ATTN_SOFTCAP
+#define ME_ATTN_SOFTCAP 0
+#endif
+// tanh through one exponential and one reciprocal: 1 - 2 / (e^(2x) + 1), exact at both ends
+__device__ __forceinline__ float fast_tanh(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * 2.8853900817779268f);
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
+}
+// Raw dot products under the cap, still to be multiplied by the scale: (cap / scale) * tanh(s * scale / cap).
+__device__ __forceinline__ void cap_scores(const AttnArgs& a, float (&sv)[8]) {
+#if ME_ATTN_SOFTCAP
+  if (a.softcap > 0.f) {
+    const float in = a.scale / a.softcap, back = a.softcap / a.scale;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sv[i] = back * fast_tanh(sv[i] * in);
+  }
+#endif
+}
+__device__ __forceinline__ float natural_lse(float m_log2, float ls) {
+  return ls > 0.f ? (m_log2 + log2f(ls)) * 0.6931471805599453f : -INFINITY;
+}
 
 // The first key a query at `pos` sees when there is a lower edge at all (a.window > 0): its block's first position
 // under a block mask, else the window's. Both grow with pos, which is all the kernels assume of it.
@@ -284,8 +311,10 @@ __device__ __forceinline__ void attend_block(const AttnArgs& a, const KVBlock& b
   float sv[8];
   float bm = NEG;
 #pragma unroll
+  for (int i = 0; i < 8; ++i) sv[i] = st[i >> 2][i & 3];
+  cap_scores(a, sv);
+#pragma unroll
   for (int i = 0; i < 8; ++i) {
-    sv[i] = st[i >> 2][i & 3];
     if (!FULL) {
       const int j = t0 + 8 * g + i;
       sv[i] = (j <= col_hi && j >= col_lo) ? sv[i] : NEG;
@@ -374,6 +403,7 @@ __device__ __forceinline__ void block_softmax(const AttnArgs& a, const f32x4 (&s
   float sv[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) sv[i] = st[i >> 2][i & 3];
+  cap_scores(a, sv);
   if (!FULL) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -576,6 +606,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         if (g == 0) { p[HD] = m[ct]; p[HD + 1] = ls; }
       } else if (valid[ct]) {
         const float inv = ls > 0.f ? 1.f / ls : 0.f;
+        if (a.lse_out != nullptr && g == 0) a.lse_out[(int64_t)tq[ct] * a.Hq + head[ct]] = natural_lse(m[ct], ls);
         bf16_t* o = a.out + tq[ct] * a.out_stride + (int64_t)head[ct] * HD + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -872,6 +903,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         if (g == 0) { p[HD] = m[ct]; p[HD + 1] = ls; }
       } else if (valid[ct]) {
         const float inv = ls > 0.f ? 1.f / ls : 0.f;
+        if (a.lse_out != nullptr && g == 0) a.lse_out[(int64_t)tq[ct] * a.Hq + head[ct]] = natural_lse(m[ct], ls);
         bf16_t* o = a.out + tq[ct] * a.out_stride + (int64_t)head[ct] * HD + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -1214,6 +1246,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(W, W))
         if (g == 0) { p[HD] = m[ct]; p[HD + 1] = ls; }
       } else if (valid[ct]) {
         const float inv = ls > 0.f ? 1.f / ls : 0.f;
+        if (a.lse_out != nullptr && g == 0) a.lse_out[(int64_t)tq[ct] * a.Hq + head[ct]] = natural_lse(m[ct], ls);
         bf16_t* o = a.out + tq[ct] * a.out_stride + (int64_t)head[ct] * HD + 4 * g;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -1269,6 +1302,7 @@ __global__ void __launch_bounds__(256) attn_prefill_merge_kernel(AttnArgs a, int
     for (int i = 0; i < MERGE_EPL; ++i) o[i] += w * v[i];
   }
   const float inv = ls > 0.f ? 1.f / ls : 0.f;
+  if (a.lse_out != nullptr && part == 0) a.lse_out[row] = natural_lse(M, ls);
   bf16_t* dst = a.out + t * a.out_stride + (int64_t)hq * HD + part * MERGE_EPL;
 #pragma unroll
   for (int i = 0; i < MERGE_EPL; ++i) dst[i] = static_cast<bf16_t>(o[i] * inv);
@@ -1524,6 +1558,7 @@ __global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
     const int hq = kvh * a.G + ctile * 16 + c;
     if (a.num_parts == 1) {
       a.out[t * a.out_stride + (int64_t)hq * HD + d] = static_cast<bf16_t>(ls > 0.f ? o / ls : 0.f);
+      if (a.lse_out != nullptr && d == 0) a.lse_out[(int64_t)t * a.Hq + hq] = natural_lse(M, ls);
     } else {
       const int64_t row = ((int64_t)b * a.Hq + hq) * a.num_parts + part;
       a.tmp_out[row * HD + d] = o;
@@ -1558,7 +1593,10 @@ __global__ void __launch_bounds__(128) attn_reduce_kernel(AttnArgs a) {
     const float f = p < P ? exp2f(mp - M) : 0.f;
     const float ls = wave_sum(f * lp);
     wgt[p] = f;
-    if (p == 0) inv_s = ls > 0.f ? 1.f / ls : 0.f;
+    if (p == 0) {
+      inv_s = ls > 0.f ? 1.f / ls : 0.f;
+      if (a.lse_out != nullptr) a.lse_out[(int64_t)b * a.Hq + hq] = natural_lse(M, ls);
+    }
   }
   __syncthreads();
   const float inv = inv_s;
@@ -1586,7 +1624,9 @@ extern "C" int me_attn_head_dim() { return HD; }
 static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, int64_t out_stride,
                        const void* k_cache, const void* v_cache, const int32_t* block_tables, int bt_stride,
                        const int32_t* context_lens, int num_seqs, int Hq, int Hkv, int page, float scale,
-                       int window) {
+                       int window, float softcap = 0.f, float* lse_out = nullptr) {
+  ME_CHECK(ME_ATTN_SOFTCAP || softcap == 0.f, "attention: this library was built without the score cap");
+  ME_CHECK(softcap >= 0.f, "attention: the score cap must not be negative");
   ME_CHECK(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0, "attention: %d query heads are not a multiple of %d key heads", Hq, Hkv);
   ME_CHECK(page >= 8 && (page & (page - 1)) == 0, "attention (bf16 MFMA path): page size %d must be a power of two, 8 or more", page);
   ME_CHECK(q_stride % 8 == 0 && out_stride % 4 == 0, "attention: token strides must keep 16-byte alignment");
@@ -1608,6 +1648,7 @@ static int fill_common(AttnArgs& a, const void* q, int64_t q_stride, void* out, 
   a.seg_keys = 0; a.max_segs = 1; a.pf_scratch = nullptr; a.seq_of_token = nullptr; a.seq_base = 0;
   a.raw_k = a.raw_v = nullptr; a.q_w = a.k_w = nullptr; a.eps = 0.f; a.rope = nullptr;
   a.k_cache_w = a.v_cache_w = nullptr;
+  a.softcap = softcap; a.lse_out = lse_out;
   return 0;
 }
 
@@ -1618,11 +1659,11 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
                                int bt_stride, const int32_t* context_lens, const int32_t* cu_seqlens,
                                int num_seqs, int64_t num_tokens, int Hq, int Hkv, int page, float scale,
                                int window, int col_tiles_per_wave, int shared, int waves, int seg_keys, int max_segs, float* pf_scratch,
-                               const int32_t* seq_of_token, int seq_base, hipStream_t stream) {
+                               const int32_t* seq_of_token, int seq_base, float softcap, float* lse_out, hipStream_t stream) {
   if (num_seqs == 0 || num_tokens == 0) return 0;
   AttnArgs a;
   if (fill_common(a, q, q_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
-                  num_seqs, Hq, Hkv, page, scale, window)) return -1;
+                  num_seqs, Hq, Hkv, page, scale, window, softcap, lse_out)) return -1;
   a.cu_seqlens = cu_seqlens;
   // column tiles per wave: 2 when the step has enough tokens to fill the GPU with the larger tiles
   const int ct = (col_tiles_per_wave == 1 || col_tiles_per_wave == 2) ? col_tiles_per_wave
@@ -1723,11 +1764,11 @@ extern "C" int me_attn_decode(const void* q, int64_t q_stride, void* out, int64_
                               const void* k_cache, const void* v_cache, const int32_t* block_tables,
                               int bt_stride, const int32_t* context_lens, int num_seqs, int Hq, int Hkv,
                               int page, float scale, int window, int part_size, int num_parts,
-                              float* scratch, int spread_heads, hipStream_t stream) {
+                              float* scratch, int spread_heads, float softcap, float* lse_out, hipStream_t stream) {
   if (num_seqs == 0) return 0;
   AttnArgs a;
   if (fill_common(a, q, q_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
-                  num_seqs, Hq, Hkv, page, scale, window)) return -1;
+                  num_seqs, Hq, Hkv, page, scale, window, softcap, lse_out)) return -1;
   return launch_decode(a, num_seqs, part_size, num_parts, scratch, spread_heads, false, stream);
 }
 
@@ -1742,11 +1783,11 @@ extern "C" int me_attn_decode_fused(const void* qkv, int64_t row_stride, void* o
                                     void* k_cache, void* v_cache, const int32_t* block_tables, int bt_stride,
                                     const int32_t* context_lens, int max_context, int num_seqs, int Hq, int Hkv,
                                     int page, float scale, int window, int part_size, int num_parts,
-                                    float* scratch, int spread_heads, hipStream_t stream) {
+                                    float* scratch, int spread_heads, float softcap, float* lse_out, hipStream_t stream) {
   if (num_seqs == 0) return 0;
   AttnArgs a;
   if (fill_common(a, qkv, row_stride, out, out_stride, k_cache, v_cache, block_tables, bt_stride, context_lens,
-                  num_seqs, Hq, Hkv, page, scale, window)) return -1;
+                  num_seqs, Hq, Hkv, page, scale, window, softcap, lse_out)) return -1;
   ME_CHECK((q_w == nullptr) == (k_w == nullptr), "attention: give both norm weights or neither");
   ME_CHECK(rope == nullptr || (max_context >= 0 && max_context <= rope_rows),
            "attention: a context of %d tokens is beyond the rotation table's %d positions", max_context, rope_rows);

@@ -146,3 +146,116 @@ extern "C" int me_attn_simple(const void* q, int64_t q_stride, void* out, int64_
   ME_LAUNCH_CHECK();
   return 0;
 }
+
+// ------------------------------------------------------------------ further terms of a softmax that another kernel has formed
+// The matrix-core kernels attend over one contiguous range of keys. What a mask or a softmax has beyond that joins here:
+// the keys at positions below keep_first that a window has left behind, and a sink per head. out holds the other
+// kernel's normalised result and lse the natural logarithm of its denominator (-inf: it saw no key). With
+// (m2, l2, acc2) the kept keys' maximum, sum and weighted values, sk the sink and M the largest of lse, m2, sk:
+//   out <- (out e^(lse - M) + acc2 e^(m2 - M)) / (e^(lse - M) + l2 e^(m2 - M) + e^(sk - M)).
+// One wave per (token, head); a lane takes a key for the scores and the channels lane, lane + 64, ... for the values.
+#define AT_MAX_D 512
+template <typename T>
+__global__ void __launch_bounds__(64)
+attn_tail_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ out, int64_t out_stride, const float* __restrict__ lse,
+                 const T* __restrict__ k_cache, const T* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int bt_stride,
+                 const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
+                 const int32_t* __restrict__ context_lens, int Hq, int Hkv, int D, int page, float scale, int window,
+                 int keep_first, float softcap, const float* __restrict__ sinks) {
+  __shared__ float qs[AT_MAX_D];
+  __shared__ float sc[64];
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const int kvh = h / (Hq / Hkv);
+  const int b = seq_of_token[t];
+  const int pos = positions[t];
+  const int32_t* bt = block_tables + (int64_t)b * bt_stride;
+  const int hi = min(pos + 1, context_lens[b]);
+  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  const int kept = (window > 0 && keep_first > 0) ? min(min(keep_first, lo), hi) : 0;
+  float m2 = -INFINITY, l2 = 0.f;
+  float acc[AT_MAX_D / 64];
+#pragma unroll
+  for (int i = 0; i < AT_MAX_D / 64; ++i) acc[i] = 0.f;
+  if (kept > 0) {
+    for (int d = lane; d < D; d += 64) qs[d] = to_f32<T>(q[t * q_stride + (int64_t)h * D + d]);
+    __syncthreads();
+    for (int c0 = 0; c0 < kept; c0 += 64) {
+      const int j = c0 + lane;
+      float s = -INFINITY;
+      if (j < kept) {
+        const int64_t pg = bt[j / page];
+        if (pg >= 0) {
+          const T* kr = k_cache + ((pg * Hkv + kvh) * (int64_t)page + j % page) * D;
+          float dot = 0.f;
+          for (int d = 0; d < D; ++d) dot += qs[d] * to_f32<T>(kr[d]);
+          s = dot * scale;
+          if (softcap > 0.f) s = softcap * tanhf(s / softcap);
+        }
+      }
+      const float m_new = fmaxf(m2, wave_max(s));
+      const float p = (s > -INFINITY) ? expf(s - m_new) : 0.f;
+      const float alpha = (m2 == -INFINITY) ? 0.f : expf(m2 - m_new);
+      l2 = l2 * alpha + wave_sum(p);
+      m2 = m_new;
+      __syncthreads();
+      sc[lane] = p;
+      __syncthreads();
+      const int je = min(64, kept - c0);
+#pragma unroll
+      for (int i = 0; i < AT_MAX_D / 64; ++i) {
+        const int d = lane + 64 * i;
+        if (d < D) {
+          float a = 0.f;
+          for (int jj = 0; jj < je; ++jj) {
+            const int64_t pg = bt[(c0 + jj) / page];
+            if (pg < 0) continue;
+            a += sc[jj] * to_f32<T>(v_cache[((pg * Hkv + kvh) * (int64_t)D + d) * page + (c0 + jj) % page]);
+          }
+          acc[i] = acc[i] * alpha + a;
+        }
+      }
+    }
+  }
+  const float l1 = lse[t * Hq + h];
+  const float sk = sinks != nullptr ? sinks[h] : -INFINITY;
+  const float M = fmaxf(fmaxf(l1, m2), sk);
+  float w1 = 0.f, w2 = 0.f, ws = 0.f;
+  if (M > -INFINITY) {
+    w1 = l1 > -INFINITY ? expf(l1 - M) : 0.f;
+    w2 = m2 > -INFINITY ? expf(m2 - M) : 0.f;
+    ws = sk > -INFINITY ? expf(sk - M) : 0.f;
+  }
+  const float denom = w1 + w2 * l2 + ws;
+  const float inv = denom > 0.f ? 1.f / denom : 0.f;
+#pragma unroll
+  for (int i = 0; i < AT_MAX_D / 64; ++i) {
+    const int d = lane + 64 * i;
+    if (d < D) {
+      T* at = out + t * out_stride + (int64_t)h * D + d;
+      *at = from_f32<T>((to_f32<T>(*at) * w1 + acc[i] * w2) * inv);
+    }
+  }
+}
+
+extern "C" int me_attn_tail(const void* q, int64_t q_stride, void* out, int64_t out_stride, const float* lse, int dtype,
+                            const void* k_cache, const void* v_cache, const int32_t* block_tables, int bt_stride,
+                            const int32_t* seq_of_token, const int32_t* positions, const int32_t* context_lens,
+                            int64_t num_tokens, int Hq, int Hkv, int D, int page, float scale, int window, int keep_first,
+                            float softcap, const float* sinks, hipStream_t stream) {
+  if (num_tokens == 0) return 0;
+  ME_CHECK(Hq >= 1 && Hkv >= 1 && Hq % Hkv == 0 && Hq <= 65535, "attention tail: %d query heads over %d key heads", Hq, Hkv);
+  ME_CHECK(D >= 1 && D <= AT_MAX_D && page >= 1 && keep_first >= 0 && softcap >= 0.f, "attention tail: head size 1..%d", AT_MAX_D);
+  ME_CHECK(lse != nullptr && num_tokens <= 2147483647ll, "attention tail: the other kernel's denominators are missing");
+  dim3 grid((unsigned)num_tokens, Hq), block(64);
+  if (dtype == ME_F32)
+    attn_tail_kernel<float><<<grid, block, 0, stream>>>((const float*)q, q_stride, (float*)out, out_stride, lse, (const float*)k_cache,
+        (const float*)v_cache, block_tables, bt_stride, seq_of_token, positions, context_lens, Hq, Hkv, D, page, scale, window,
+        keep_first, softcap, sinks);
+  else
+    attn_tail_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, lse, (const bf16_t*)k_cache,
+        (const bf16_t*)v_cache, block_tables, bt_stride, seq_of_token, positions, context_lens, Hq, Hkv, D, page, scale, window,
+        keep_first, softcap, sinks);
+  ME_LAUNCH_CHECK();
+  return 0;
+}

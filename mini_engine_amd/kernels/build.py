@@ -34,6 +34,7 @@ ATTN_SOURCE = "attention_mfma.hip"
 HEADERS = ["common.h", "errors.inc", "sampling.h"]
 # Head sizes that build_all() compiles ahead of use; any other multiple of 16 up to 512 is compiled when a model first needs it.
 DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
+CAPPED_HEAD_DIMS = (32, 64, 128)          # ... of the variant with a cap on the scores
 
 _locks: dict = {}
 _locks_guard = threading.Lock()
@@ -187,9 +188,13 @@ def core_library(force: bool = False) -> str:
     return _ensure("libme_core.so", CORE_SOURCES, [], force)
 
 
-def attention_library(head_dim: int, force: bool = False) -> str:
+def attention_library(head_dim: int, force: bool = False, score_cap: bool = False) -> str:
+    """The matrix-core attention kernels for one head size. `score_cap`: the variant whose softmax bends its scores under
+    a cap first (a library of its own, so that the kernels of models without a cap stay as they are)."""
     if head_dim % 16 or not 16 <= head_dim <= 512:
         raise BuildError(f"the bf16 attention kernels need a head size that is a multiple of 16 in 16..512, got {head_dim}")
+    if score_cap:
+        return _ensure(f"libme_attn_d{head_dim}c.so", [ATTN_SOURCE], [f"-DME_HEAD_DIM={head_dim}", "-DME_ATTN_SOFTCAP=1"], force)
     return _ensure(f"libme_attn_d{head_dim}.so", [ATTN_SOURCE], [f"-DME_HEAD_DIM={head_dim}"], force)
 
 
@@ -198,4 +203,5 @@ def build_all(head_dims=DEFAULT_HEAD_DIMS, force: bool = True) -> list:
     libs = [core_library(force=force)]
     with ThreadPoolExecutor(max_workers=4) as pool:
         libs += list(pool.map(lambda d: attention_library(d, force=force), head_dims))
+        libs += list(pool.map(lambda d: attention_library(d, force=force, score_cap=True), CAPPED_HEAD_DIMS))
     return libs

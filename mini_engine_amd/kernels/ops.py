@@ -65,6 +65,7 @@ _CORE_PROTOS = {
     "me_qk_norm_rope_store": [P, I, L, L, P, P, F, P, L, L, P, P, P, P, I, I, I, I, I, P],
     "me_store_kv": [P, P, I, L, L, L, P, P, P, I, I, I, P],
     "me_attn_simple": [P, L, P, L, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, I, F, P, P],
+    "me_attn_tail": [P, L, P, L, P, I, P, P, P, I, P, P, P, L, I, I, I, I, F, I, I, F, P, P],
     "me_gemm_tiled": [P, L, P, L, P, L, I, I, I, I, I, P],
     "me_gemm_skinny_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, I, I, P],
     "me_gemm_rows_bf16": [P, L, P, L, P, L, I, P, I, I, I, I, I, P],
@@ -96,9 +97,9 @@ _CORE_PROTOS = {
     "me_sample_static": [P, L, P, P, P, I, I, P],
 }
 _ATTN_PROTOS = {
-    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, I, P, P, I, P],
-    "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, I, P],
-    "me_attn_decode_fused": [P, L, P, L, P, P, F, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, I, P],
+    "me_attn_prefill": [P, L, P, L, P, P, P, I, P, P, I, L, I, I, I, F, I, I, I, I, I, I, P, P, I, F, P, P],
+    "me_attn_decode": [P, L, P, L, P, P, P, I, P, I, I, I, I, F, I, I, I, P, I, F, P, P],
+    "me_attn_decode_fused": [P, L, P, L, P, P, F, P, I, P, P, P, I, P, I, I, I, I, I, F, I, I, I, P, I, F, P, P],
 }
 
 _core: _Lib | None = None
@@ -119,15 +120,16 @@ def core() -> _Lib:
     return _core
 
 
-def attn_lib(head_dim: int) -> _Lib:
-    lib = _attn.get(head_dim)
+def attn_lib(head_dim: int, score_cap: bool = False) -> _Lib:
+    key = (head_dim, bool(score_cap)) if score_cap else head_dim
+    lib = _attn.get(key)
     if lib is None:
         _require_gpu()
-        lib = _Lib(build.attention_library(head_dim), _ATTN_PROTOS)
+        lib = _Lib(build.attention_library(head_dim, score_cap=bool(score_cap)), _ATTN_PROTOS)
         lib.cdll.me_attn_head_dim.restype = c_int
         if lib.cdll.me_attn_head_dim() != head_dim:
             raise KernelError(f"{lib.path} was built for head size {lib.cdll.me_attn_head_dim()}, not {head_dim}")
-        _attn[head_dim] = lib
+        _attn[key] = lib
     return lib
 
 
@@ -353,7 +355,9 @@ class HipBackend:
         floor(i / chunk) (the kernels take it as a negative window). `keep_first`: behind a window the keys j <
         keep_first stay visible. `softcap` c: every score becomes c * tanh(score / c) before the softmax. `sinks`
         (float32 [Hq]): exp(sink_h) joins the softmax's denominator of head h, a term without key or value. With any
-        of the three the rows take the exact kernel (`attn_simple`), whatever their dtype.
+        three. On the matrix-core path the cap runs inside the kernels (a library variant of its own), which also leave
+        the logarithm of every softmax denominator; a second kernel (`attn_tail`) then joins the kept keys behind the
+        window and the sink to that softmax. The float32 path and odd sizes take the exact kernel (`attn_simple`) for all of it.
 
         q: [T, Hq*D] (a strided view is fine). Rows are ordered decode requests first (one token
         each, `num_decodes` of them), then the others; `prefill_cu` int32 [B - num_decodes + 1]
@@ -383,16 +387,18 @@ class HipBackend:
         _check(not keep_first or (window and keep_first > 0), "attention: keys are kept behind a window only")
         _check(sinks is None or (sinks.dtype == torch.float32 and sinks.shape == (Hq,) and sinks.is_contiguous()),
                "attention: sinks must be float32 [Hq]")
-        plain_scores = not keep_first and not softcap and sinks is None
+        tail = bool(keep_first) or sinks is not None
         mfma = (q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 512 and page >= 8 and page & (page - 1) == 0
-                and not force_simple and plain_scores)
+                and not force_simple and (MFMA_WITH_EXTRAS or not (tail or softcap)))
         if not mfma:
             core().call("me_attn_simple", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), _code(q.dtype),
                         k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
                         seq_of_token.data_ptr(), positions.data_ptr(), context_lens.data_ptr(), T, Hq, Hkv, D, page,
                         float(scale), win, int(keep_first or 0), float(softcap or 0.0), _ptr(sinks), _stream())
             return out
-        lib = attn_lib(D)
+        lib = attn_lib(D, score_cap=bool(softcap))
+        cap = float(softcap or 0.0)
+        lse = torch.empty((T, Hq), dtype=torch.float32, device=q.device) if tail else None
         es = q.element_size()
         if (decode_as_prefill or DECODE_AS_PREFILL) and num_decodes > 0:
             ones = torch.arange(num_decodes + 1, dtype=torch.int32, device=q.device)
@@ -405,7 +411,7 @@ class HipBackend:
             lib.call("me_attn_decode", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
                      num_decodes, Hq, Hkv, page, float(scale), win, part_size, num_parts, _ptr(scratch),
-                     0 if even_contexts else 1, _stream())
+                     0 if even_contexts else 1, cap, _ptr(lse), _stream())
         if T > num_decodes:
             _check(prefill_cu is not None and _is_i32(prefill_cu, B - num_decodes + 1), "attention: prefill_cu must be int32 [B-Dn+1]")
             Tp = T - num_decodes
@@ -420,7 +426,13 @@ class HipBackend:
                      v_cache.data_ptr(), block_tables.data_ptr() + num_decodes * block_tables.stride(0) * 4,
                      block_tables.stride(0), context_lens.data_ptr() + num_decodes * 4, prefill_cu.data_ptr(),
                      B - num_decodes, Tp, Hq, Hkv, page, float(scale), win, col_tiles, PREFILL_THROUGH_LDS, waves, seg_keys, max_segs,
-                     _ptr(pf), seq_of_token.data_ptr() + num_decodes * 4, num_decodes, _stream())
+                     _ptr(pf), seq_of_token.data_ptr() + num_decodes * 4, num_decodes, cap,
+                     None if lse is None else lse.data_ptr() + num_decodes * Hq * 4, _stream())
+        if tail:
+            core().call("me_attn_tail", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), lse.data_ptr(), _code(q.dtype),
+                        k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
+                        seq_of_token.data_ptr(), positions.data_ptr(), context_lens.data_ptr(), T, Hq, Hkv, D, page, float(scale),
+                        win, int(keep_first or 0), cap, _ptr(sinks), _stream())
         return out
 
     def decode_step_attention(self, qkv, q_weight, k_weight, eps, table, k_cache, v_cache, page: int, block_tables,
@@ -460,7 +472,7 @@ class HipBackend:
                          k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
                          context_lens.data_ptr(), int(max_context), B, Hq, Hkv, page, float(scale),
                          -int(chunk) if chunk else int(window or 0),
-                         part_size, num_parts, _ptr(scratch), 0 if even_contexts else 1, _stream())
+                         part_size, num_parts, _ptr(scratch), 0 if even_contexts else 1, 0.0, None, _stream())
         return out
 
     # -- matrix products -----------------------------------------------------------------
@@ -1043,6 +1055,7 @@ PREFILL_SEGMENT_KEYS = None    # None: chosen by prefill_segments(); an int forc
 # by the loads themselves at head size 128 and pages of 16 keys or more), 2 as 1 but always staged through registers
 PREFILL_THROUGH_LDS = 1
 PREFILL_COL_TILES = 0     # 0: chosen by prefill_col_tiles(); 1 or 2 force the column tiles per wave
+MFMA_WITH_EXTRAS = True        # False: attention with kept first keys, a score cap or sinks always takes the exact kernel
 DECODE_AS_PREFILL = False      # True: single-token rows go through the prefill kernel (cross-check of the decode kernel)
 USE_MID_PRODUCT = True          # False: products of 33-512 rows over small weights go to the library like the larger ones
 MID_MAX_WEIGHT = 8 << 20

@@ -108,6 +108,7 @@ class ShiftedDecay(Mixer):
         self.add_param("u", ParamSpec((num_heads, key_dim), init=_bonus, dtype="float32"))
         self.add_param("norm_weight", ParamSpec((self.inner,), init="norm", dtype="float32"))
         self.add_child("o", Linear(self.inner, hidden_size))
+        self.value_dim = key_dim
         self.matrix_floats = num_heads * key_dim * key_dim
 
     def state_need(self):

