@@ -227,9 +227,12 @@ extern "C" int me_token_shift(const void* x, int64_t x_stride, int dtype, const 
 //                    y_p = sum_n S[n, p] q_n
 // With `unit`: q and k are first divided by sqrt(sum of their squares + unit_eps) per head; q is multiplied by q_scale.
 // Every sum runs over n only, so a column p of the state never meets another: a wave takes 64 / RG columns of one head
-// and a lane NR / RG of a column's rows, kept in registers for the whole walk; with RG > 1 the RG lanes of a column
-// add their partial sums through the lanes' exchange. q, k and the decays of a token, which all columns share, are
-// formed once per wave in LDS; the next token's raw values are on their way while the current token is worked on.
+// and a lane NR / RG of a column's rows, kept in registers for the whole walk; with RG > 1 the RG lanes of a column,
+// neighbours in the wave, add their partial sums by exchanges inside a row of 16 lanes. q, k and the decays of a token, which all columns share, are
+// formed once per wave in LDS, eight tokens at a time into one of two buffers; the next eight tokens' raw values are on
+// their way while the current eight are worked on, so a wave waits for memory once per eight tokens. The products
+// and sums of the walk are written as explicit fused multiply-adds: a token's result then does not depend on its place
+// among the eight (the compiler is free to fuse each unrolled copy otherwise).
 struct DrArgs {
   const void* q; const void* k; const void* v; const void* raw; const void* beta;
   int64_t q_stride, k_stride, v_stride, raw_stride, beta_stride;
@@ -241,12 +244,91 @@ struct DrArgs {
   int unit; float unit_eps, q_scale;
 };
 
-template <typename TX, int NR, int RG, int RULE>
-__global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a) {
+#define DR_TB 8          // tokens whose shared values are formed at once and wait in LDS
+
+// Sum over the RG neighbouring lanes that share a state column (RG 1, 4 or 16, aligned groups), left in all of them: lane
+// exchanges inside a row of 16 lanes (quad permutations, then rotations of the row), no trip through LDS.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int RG>
+__device__ __forceinline__ float group_sum(float v) {
+  if (RG >= 2) v += dpp_f<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  if (RG >= 4) v += dpp_f<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  if (RG >= 8) v += dpp_f<0x124>(v);     // row_ror 4
+  if (RG >= 16) v += dpp_f<0x128>(v);    // row_ror 8
+  return v;
+}
+
+// What a token's q, k, raw decay and write strength become before the recurrence reads them, for one wave that holds
+// rows lane, lane + 64, ... of one head: q and k at unit length and scaled, the decay, and the token's own number
+// (sigmoid(beta), or sum_n q_n bonus_n k_n under the bonus rule), which every lane gets.
+template <int PER, int RULE>
+__device__ __forceinline__ float shape_token(const DrArgs& a, int lane, int nr_rows, float (&q)[PER], float (&k)[PER], float (&d)[PER],
+                                             const float (&base)[PER], const float (&bonus)[PER], float rate, float beta) {
+  float qs = a.q_scale, ks = 1.0f;
+  if (a.unit) {
+    float q2 = 0.f, k2 = 0.f;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) { q2 += q[i] * q[i]; k2 += k[i] * k[i]; }
+    qs = a.q_scale / sqrtf(wave_sum(q2) + a.unit_eps);
+    ks = 1.0f / sqrtf(wave_sum(k2) + a.unit_eps);
+  }
+  float own = 0.f;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int n = lane + 64 * i;
+    q[i] *= qs;
+    k[i] *= ks;
+    float dv;
+    if (RULE == 0) dv = expf(-expf(d[i] + base[i]));
+    else dv = expf(-rate * hy_softplus(d[i] + base[i]));
+    d[i] = (n < a.N && n < nr_rows) ? dv : 1.0f;
+    own += q[i] * bonus[i] * k[i];
+  }
+  return RULE == 1 ? hy_sigmoid(beta) : wave_sum(own);
+}
+
+// One wave per (token, head): the shaped values of every token at once, for a recurrence kernel that then only streams
+// them (PRE): pre_q, pre_k, pre_d [T, H, NR] and pre_x [T, H], float32.
+template <typename TX, int NR, int RULE>
+__global__ void __launch_bounds__(64) decay_prepare_kernel(DrArgs a, float* __restrict__ pre_q, float* __restrict__ pre_k,
+                                                           float* __restrict__ pre_d, float* __restrict__ pre_x) {
+  constexpr int PER = (NR + 63) / 64;
+  const int64_t t = blockIdx.x;
+  const int h = blockIdx.y, lane = threadIdx.x;
+  const int g = h / (a.H / a.G);
+  const TX* qp = (const TX*)a.q; const TX* kp = (const TX*)a.k; const TX* rp = (const TX*)a.raw; const TX* bp = (const TX*)a.beta;
+  float q[PER], k[PER], d[PER], base[PER], bonus[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int n = lane + 64 * i;
+    const bool in = n < a.N && n < NR;
+    base[i] = in ? a.base[h * a.N + n] : 0.f;
+    bonus[i] = (RULE == 0 && in) ? a.bonus[h * a.N + n] : 0.f;
+    q[i] = in ? to_f32<TX>(qp[t * a.q_stride + g * a.N + n]) : 0.f;
+    k[i] = in ? to_f32<TX>(kp[t * a.k_stride + g * a.N + n]) : 0.f;
+    d[i] = in ? to_f32<TX>(rp[t * a.raw_stride + h * a.N + n]) : 0.f;
+  }
+  const float beta = RULE == 1 ? to_f32<TX>(bp[t * a.beta_stride + h]) : 0.f;
+  const float x = shape_token<PER, RULE>(a, lane, NR, q, k, d, base, bonus, RULE == 1 ? a.rate[h] : 0.f, beta);
+  const int64_t at = (t * a.H + h) * NR;
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const int n = lane + 64 * i;
+    if (n < NR) { pre_q[at + n] = q[i]; pre_k[at + n] = k[i]; pre_d[at + n] = d[i]; }
+  }
+  if (lane == 0) pre_x[t * a.H + h] = x;
+}
+
+template <typename TX, int NR, int RG, int RULE, bool PRE>
+__global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a, const float* __restrict__ pre_q, const float* __restrict__ pre_k,
+                                                        const float* __restrict__ pre_d, const float* __restrict__ pre_x) {
   constexpr int PC = 64 / RG;            // columns per wave
   constexpr int RL = NR / RG;            // rows per lane
-  constexpr int PER = (NR + 63) / 64;    // rows of q, k and the decay that a lane forms for the wave
-  __shared__ float sq[NR], sk[NR], sd[NR];
+  constexpr int PER = (NR + 63) / 64;    // rows of q, k and the decay that a lane brings to LDS for the wave
+  __shared__ float sq[2][DR_TB][NR], sk[2][DR_TB][NR], sd[2][DR_TB][NR];
   const int lane = threadIdx.x;
   const int col_blocks = (a.P + PC - 1) / PC;
   const int cb = blockIdx.x % col_blocks;
@@ -256,14 +338,16 @@ __global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a) {
   const int64_t first = a.cu[b];
   const int n_tok = (int)(a.cu[b + 1] - first);
   if (n_tok <= 0) return;
-  const int p = cb * PC + lane % PC;
-  const int r0 = (lane / PC) * RL;
+  // the RG lanes of a column are neighbours; lane rg of them keeps rows rg, rg + RG, ... (neighbours read neighbouring
+  // words of LDS, the lanes of the wave's other columns the same words)
+  const int p = cb * PC + lane / RG;
+  const int rg = lane % RG;
   const bool live = p < a.P;
   const int pc = live ? p : a.P - 1;
   float* srow = a.state + (int64_t)a.slots[b] * a.state_stride + (int64_t)h * a.N * a.P;
   float S[RL];
 #pragma unroll
-  for (int i = 0; i < RL; ++i) S[i] = (r0 + i < a.N) ? srow[(int64_t)(r0 + i) * a.P + pc] : 0.f;
+  for (int i = 0; i < RL; ++i) S[i] = (i * RG + rg < a.N) ? srow[(int64_t)(i * RG + rg) * a.P + pc] : 0.f;
 
   const TX* qp = (const TX*)a.q; const TX* kp = (const TX*)a.k; const TX* vp = (const TX*)a.v;
   const TX* rp = (const TX*)a.raw; const TX* bp = (const TX*)a.beta;
@@ -271,127 +355,136 @@ __global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a) {
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
     const int n = lane + 64 * i;
-    const bool in = n < a.N && n < NR;
+    const bool in = !PRE && n < a.N && n < NR;
     base[i] = in ? a.base[h * a.N + n] : 0.f;
     bonus[i] = (RULE == 0 && in) ? a.bonus[h * a.N + n] : 0.f;
   }
-  const float rate = RULE == 1 ? a.rate[h] : 0.f;
-  float nq[PER], nk[PER], nr[PER], nv, nb = 0.f;
-  auto fetch = [&](int t) {
-    const int64_t row = first + t;
+  const float rate = (RULE == 1 && !PRE) ? a.rate[h] : 0.f;
+  // a batch of tokens on its way (n*) and the batch being worked on (c*): a lane's own column's v and the token's own
+  // number (the write strength, or under the bonus rule sum_n q_n bonus_n k_n)
+  float nq[DR_TB][PER], nk[DR_TB][PER], nr[DR_TB][PER], nv[DR_TB], nb[DR_TB];
+  float cv[DR_TB], cx[DR_TB];
+  auto fetch = [&](int t0) {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int n = lane + 64 * i;
-      const bool in = n < a.N && n < NR;
-      nq[i] = in ? to_f32<TX>(qp[row * a.q_stride + g * a.N + n]) : 0.f;
-      nk[i] = in ? to_f32<TX>(kp[row * a.k_stride + g * a.N + n]) : 0.f;
-      nr[i] = in ? to_f32<TX>(rp[row * a.raw_stride + h * a.N + n]) : 0.f;
+    for (int j = 0; j < DR_TB; ++j) {
+      if (t0 + j < n_tok) {
+        const int64_t row = first + t0 + j;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int n = lane + 64 * i;
+          if (PRE) {
+            const int64_t at = (row * a.H + h) * NR + (n < NR ? n : 0);
+            nq[j][i] = pre_q[at]; nk[j][i] = pre_k[at]; nr[j][i] = pre_d[at];
+          } else {
+            const bool in = n < a.N && n < NR;
+            nq[j][i] = in ? to_f32<TX>(qp[row * a.q_stride + g * a.N + n]) : 0.f;
+            nk[j][i] = in ? to_f32<TX>(kp[row * a.k_stride + g * a.N + n]) : 0.f;
+            nr[j][i] = in ? to_f32<TX>(rp[row * a.raw_stride + h * a.N + n]) : 0.f;
+          }
+        }
+        nv[j] = to_f32<TX>(vp[row * a.v_stride + h * a.P + pc]);
+        if (PRE) nb[j] = pre_x[row * a.H + h];
+        else nb[j] = RULE == 1 ? to_f32<TX>(bp[row * a.beta_stride + h]) : 0.f;
+      }
     }
-    nv = to_f32<TX>(vp[row * a.v_stride + h * a.P + pc]);
-    if (RULE == 1) nb = to_f32<TX>(bp[row * a.beta_stride + h]);
+  };
+  // the fetched batch's shared values into LDS buffer `buf`, its per-lane values into c*
+  auto settle = [&](int t0, int buf) {
+#pragma unroll
+    for (int j = 0; j < DR_TB; ++j) {
+      if (t0 + j < n_tok) {
+        float x = nb[j];
+        if (!PRE) x = shape_token<PER, RULE>(a, lane, NR, nq[j], nk[j], nr[j], base, bonus, rate, nb[j]);
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+          const int n = lane + 64 * i;
+          if (n < NR) { sq[buf][j][n] = nq[j][i]; sk[buf][j][n] = nk[j][i]; sd[buf][j][n] = nr[j][i]; }
+        }
+        cv[j] = nv[j];
+        cx[j] = x;
+      }
+    }
   };
   fetch(0);
-  for (int t = 0; t < n_tok; ++t) {
-    // this token's shared values into LDS
-    float qs = 0.f, ks = 0.f;
-    if (a.unit) {
+  for (int t0 = 0, buf = 0; t0 < n_tok; t0 += DR_TB, buf ^= 1) {
+    settle(t0, buf);
+    __syncthreads();      // the batch is in LDS; the other buffer, which the next batch will take, has been read by all
+    if (t0 + DR_TB < n_tok) fetch(t0 + DR_TB);
 #pragma unroll
-      for (int i = 0; i < PER; ++i) { qs += nq[i] * nq[i]; ks += nk[i] * nk[i]; }
-      qs = wave_sum(qs); ks = wave_sum(ks);
-      qs = a.q_scale / sqrtf(qs + a.unit_eps);
-      ks = 1.0f / sqrtf(ks + a.unit_eps);
-    } else {
-      qs = a.q_scale; ks = 1.0f;
-    }
-    __syncthreads();                     // the token before has been read by every lane
+    for (int j = 0; j < DR_TB; ++j) {
+      if (t0 + j < n_tok) {
+        const float v = cv[j];
+        float y = 0.f;
+        if (RULE == 0) {
 #pragma unroll
-    for (int i = 0; i < PER; ++i) {
-      const int n = lane + 64 * i;
-      if (n < NR) {
-        const bool in = n < a.N;
-        sq[n] = nq[i] * qs;
-        sk[n] = nk[i] * ks;
-        float d;
-        if (RULE == 0) d = expf(-expf(nr[i] + base[i]));
-        else d = expf(-rate * hy_softplus(nr[i] + base[i]));
-        sd[n] = in ? d : 1.0f;
+          for (int i = 0; i < RL; ++i) {
+            const int n = i * RG + rg;
+            y = fmaf(sq[buf][j][n], S[i], y);
+            S[i] = fmaf(sd[buf][j][n], S[i], sk[buf][j][n] * v);
+          }
+        } else {
+          float dot = 0.f;
+#pragma unroll
+          for (int i = 0; i < RL; ++i) {
+            const int n = i * RG + rg;
+            S[i] *= sd[buf][j][n];
+            dot = fmaf(S[i], sk[buf][j][n], dot);
+          }
+          dot = group_sum<RG>(dot);
+          const float u = cx[j] * (v - dot);
+#pragma unroll
+          for (int i = 0; i < RL; ++i) {
+            const int n = i * RG + rg;
+            S[i] = fmaf(sk[buf][j][n], u, S[i]);
+            y = fmaf(S[i], sq[buf][j][n], y);
+          }
+        }
+        y = group_sum<RG>(y);
+        if (RULE == 0) y = fmaf(cx[j], v, y);       // the current token's own term: v_p * sum_n q_n bonus_n k_n
+        if (live && rg == 0) a.y[(first + t0 + j) * (int64_t)(a.H * a.P) + h * a.P + p] = y;
       }
     }
-    const float v = nv;
-    const float beta = RULE == 1 ? hy_sigmoid(nb) : 0.f;
-    float bon[PER];
-#pragma unroll
-    for (int i = 0; i < PER; ++i) bon[i] = bonus[i];
-    __syncthreads();
-    if (t + 1 < n_tok) fetch(t + 1);
-    float y = 0.f;
-    if (RULE == 0) {
-#pragma unroll
-      for (int i = 0; i < RL; ++i) {
-        const int n = r0 + i;
-        const float kv = sk[n] * v;
-        // the bonus of row n: kept by lane n % 64 of the wave; every lane needs the rows of its own slice
-        y += sq[n] * S[i];
-        S[i] = sd[n] * S[i] + kv;
-      }
-    } else {
-      float dot = 0.f;
-#pragma unroll
-      for (int i = 0; i < RL; ++i) {
-        const int n = r0 + i;
-        S[i] *= sd[n];
-        dot += S[i] * sk[n];
-      }
-#pragma unroll
-      for (int off = PC; off < 64; off <<= 1) dot += __shfl_xor(dot, off, ME_WAVE);
-      const float u = beta * (v - dot);
-#pragma unroll
-      for (int i = 0; i < RL; ++i) {
-        const int n = r0 + i;
-        S[i] += sk[n] * u;
-        y += S[i] * sq[n];
-      }
-    }
-#pragma unroll
-    for (int off = PC; off < 64; off <<= 1) y += __shfl_xor(y, off, ME_WAVE);
-    if (RULE == 0) {
-      // the current token's own term: v_p * sum_n q_n bonus_n k_n, one number per wave
-      float own = 0.f;
-#pragma unroll
-      for (int i = 0; i < PER; ++i) { const int n = lane + 64 * i; if (n < NR) own += sq[n] * bon[i] * sk[n]; }
-      own = wave_sum(own);
-      y += own * v;
-    }
-    if (live && lane < PC) a.y[(first + t) * (int64_t)(a.H * a.P) + h * a.P + p] = y;
   }
   if (live) {
 #pragma unroll
     for (int i = 0; i < RL; ++i)
-      if (r0 + i < a.N) srow[(int64_t)(r0 + i) * a.P + p] = S[i];
+      if (i * RG + rg < a.N) srow[(int64_t)(i * RG + rg) * a.P + p] = S[i];
   }
 }
 
-template <typename TX, int NR, int RG>
-static void launch_decay_rows(const DrArgs& a, int rule, int num_seqs, hipStream_t stream) {
+template <typename TX, int NR, int RG, bool PRE>
+static void launch_decay_rows(const DrArgs& a, int rule, int num_seqs, int64_t T, float* pre, hipStream_t stream) {
   constexpr int PC = 64 / RG;
   const dim3 grid((unsigned)(num_seqs * a.H * ((a.P + PC - 1) / PC))), block(64);
-  if (rule == 0) decay_rows_kernel<TX, NR, RG, 0><<<grid, block, 0, stream>>>(a);
-  else decay_rows_kernel<TX, NR, RG, 1><<<grid, block, 0, stream>>>(a);
+  float* pq = pre; float* pk = pre; float* pd = pre; float* px = pre;
+  if (PRE) {
+    const int64_t each = T * a.H * NR;
+    pk = pre + each; pd = pre + 2 * each; px = pre + 3 * each;
+    const dim3 pgrid((unsigned)T, a.H);
+    if (rule == 0) decay_prepare_kernel<TX, NR, 0><<<pgrid, block, 0, stream>>>(a, pq, pk, pd, px);
+    else decay_prepare_kernel<TX, NR, 1><<<pgrid, block, 0, stream>>>(a, pq, pk, pd, px);
+  }
+  if (rule == 0) decay_rows_kernel<TX, NR, RG, 0, PRE><<<grid, block, 0, stream>>>(a, pq, pk, pd, px);
+  else decay_rows_kernel<TX, NR, RG, 1, PRE><<<grid, block, 0, stream>>>(a, pq, pk, pd, px);
 }
 
-// row_groups: lanes that share a column (1 or 4); 4 gives four times the waves with a quarter of the rows each.
+// row_groups: lanes that share a column: 1 or 4 (4 gives four times the waves with a quarter of the rows each) with the
+// tokens' values shaped inside the kernel; 4 or 16 with `pre`, scratch of 3 T H NR + T H floats (NR: N rounded up to 32, 64,
+// 128 or 256) that a first kernel fills with the shaped values of all tokens at once, so that the walk only streams them.
 extern "C" int me_decay_rows_recurrence(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                                         const void* raw, int64_t raw_stride, const void* beta, int64_t beta_stride, int dtype,
                                         const float* base, const float* rate, const float* bonus, float* state, int64_t state_stride,
                                         const int32_t* slots, const int32_t* cu, float* y, int num_seqs, int H, int G, int N, int P,
-                                        int rule, int unit, float unit_eps, float q_scale, int row_groups, hipStream_t stream) {
+                                        int rule, int unit, float unit_eps, float q_scale, int row_groups, int64_t T, float* pre, hipStream_t stream) {
   if (num_seqs == 0) return 0;
   ME_CHECK(H >= 1 && G >= 1 && H % G == 0 && N >= 1 && N <= 256 && P >= 1, "decay_rows_recurrence: %d heads over %d groups, state %d x %d "
            "(up to 256 rows)", H, G, N, P);
   ME_CHECK(rule == 0 || rule == 1, "decay_rows_recurrence: unknown rule %d", rule);
   ME_CHECK(rule == 0 ? bonus != nullptr : (rate != nullptr && beta != nullptr), "decay_rows_recurrence: the rule's constants are missing");
-  ME_CHECK(row_groups == 1 || row_groups == 4, "decay_rows_recurrence: 1 or 4 lanes to a column");
-  ME_CHECK((int64_t)num_seqs * H * ((P + 15) / 16) <= 2147483647ll, "decay_rows_recurrence: too many workgroups");
+  ME_CHECK(pre == nullptr ? (row_groups == 1 || row_groups == 4) : (row_groups == 4 || row_groups == 16),
+           "decay_rows_recurrence: 1 or 4 lanes to a column, 4 or 16 over prepared values");
+  ME_CHECK(T >= 0 && T <= 2147483647ll && H <= 65535, "decay_rows_recurrence: too many tokens or heads");
+  ME_CHECK((int64_t)num_seqs * H * ((P + 3) / 4) <= 2147483647ll, "decay_rows_recurrence: too many workgroups");
   DrArgs a;
   a.q = q; a.k = k; a.v = v; a.raw = raw; a.beta = beta;
   a.q_stride = q_stride; a.k_stride = k_stride; a.v_stride = v_stride; a.raw_stride = raw_stride; a.beta_stride = beta_stride;
@@ -399,8 +492,10 @@ extern "C" int me_decay_rows_recurrence(const void* q, int64_t q_stride, const v
   a.H = H; a.G = G; a.N = N; a.P = P; a.unit = unit; a.unit_eps = unit_eps; a.q_scale = q_scale;
 #define DR_NR(TX, NR)                                                           \
   do {                                                                          \
-    if (row_groups == 4) launch_decay_rows<TX, NR, 4>(a, rule, num_seqs, stream); \
-    else launch_decay_rows<TX, NR, 1>(a, rule, num_seqs, stream);               \
+    if (pre != nullptr && row_groups == 16) launch_decay_rows<TX, NR, 16, true>(a, rule, num_seqs, T, pre, stream); \
+    else if (pre != nullptr) launch_decay_rows<TX, NR, 4, true>(a, rule, num_seqs, T, pre, stream);                 \
+    else if (row_groups == 4) launch_decay_rows<TX, NR, 4, false>(a, rule, num_seqs, T, pre, stream);               \
+    else launch_decay_rows<TX, NR, 1, false>(a, rule, num_seqs, T, pre, stream);                                    \
   } while (0)
 #define DR(TX)                            \
   do {                                    \

@@ -92,7 +92,7 @@ _CORE_PROTOS = {
     "me_glu_clamped": [P, L, P, I, L, I, F, F, P],
     "me_weighted_sum": [I, P, P, P, P, P, P, P, P, F, P, P, P, I, L, I, P],
     "me_token_shift": [P, L, I, P, I, P, L, P, P, P, P, L, I, P],
-    "me_decay_rows_recurrence": [P, L, P, L, P, L, P, L, P, L, I, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, F, F, I, P],
+    "me_decay_rows_recurrence": [P, L, P, L, P, L, P, L, P, L, I, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, F, F, I, L, P, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
     "me_sample_static": [P, L, P, P, P, I, I, P],
 }
@@ -925,11 +925,14 @@ class HipBackend:
         _check(_is_i32(state_slots) and _is_i32(cu_seqlens, B + 1) and len(q_lens) == B and sum(q_lens) == T, "decay_rows_recurrence: metadata")
         _check(1 <= N <= 256 and H % G == 0, "decay_rows_recurrence: up to 256 state rows, heads a multiple of the groups")
         y = torch.empty((T, H * P), dtype=torch.float32, device=v.device)
+        groups, prepared = decay_row_groups(B, H, N, P, max(q_lens))
+        NR = 32 if N <= 32 else 64 if N <= 64 else 128 if N <= 128 else 256
+        pre = _scratch(3 * T * H * NR + T * H, v.device, "decay_rows") if prepared else None
         core().call("me_decay_rows_recurrence", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0),
                     raw.data_ptr(), raw.stride(0), _ptr(beta), 0 if beta is None else beta.stride(0), _code(dtype),
                     base.data_ptr(), _ptr(rate), _ptr(bonus), state.data_ptr(), state.stride(0), state_slots.data_ptr(),
                     cu_seqlens.data_ptr(), y.data_ptr(), B, H, G, N, P, DECAY_RULES[rule], int(unit_eps is not None),
-                    float(unit_eps or 0.0), float(q_scale), decay_row_groups(B, H, N, P), _stream())
+                    float(unit_eps or 0.0), float(q_scale), groups, T, _ptr(pre), _stream())
         return y
 
     # -- routed experts ------------------------------------------------------------------
@@ -1498,13 +1501,21 @@ def expert_tile_rows(T: int, top: int, E: int) -> int:
     return 128 if T * top >= EXPERT_LARGE_TILE_ROWS * E else 64
 
 
-def decay_row_groups(num_seqs: int, H: int, N: int, P: int) -> int:
-    """Lanes that share a column of the state in `decay_rows_recurrence`: 4 (a quarter of the rows per lane, four times the
-    waves) where a lane could not keep a whole column in registers, or while one lane to a column leaves compute units
-    without a wave; else 1 (no exchange between lanes)."""
+DECAY_PREPARE_MIN_TOKENS = 9      # requests of this many tokens or more: the tokens' values are shaped by a kernel of its own
+
+
+def decay_row_groups(num_seqs: int, H: int, N: int, P: int, longest: int = 1) -> tuple:
+    """(lanes that share a column of the state in `decay_rows_recurrence`, whether a first kernel shapes the tokens' values).
+    A request is a chain: the fewer rows a lane walks per token, the shorter the chain's step, at the price of more waves
+    and an exchange between lanes. Steps of long requests: the values of all tokens are shaped at once by a kernel of its
+    own (unit lengths, decays and their exponentials leave the chain), and 16 lanes share a column while that keeps the
+    launch within 16 waves a compute unit, else 4. Short steps shape inside the kernel: 4 lanes where a lane could not
+    keep a whole column in registers, or while one lane to a column leaves compute units without a wave; else 1."""
+    if longest >= DECAY_PREPARE_MIN_TOKENS:
+        return (16 if num_seqs * H * -(-P // 4) <= 16 * _COMPUTE_UNITS else 4), True
     if N > 64:
-        return 4
-    return 4 if num_seqs * H * -(-P // 64) < 2 * _COMPUTE_UNITS and N >= 16 else 1
+        return 4, False
+    return (4 if num_seqs * H * -(-P // 64) < 2 * _COMPUTE_UNITS and N >= 16 else 1), False
 
 
 def gated_linear_rows(rows: int, w: torch.Tensor) -> bool:

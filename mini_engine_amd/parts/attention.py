@@ -301,5 +301,8 @@ class Attention(Mixer):
             ops.sigmoid_gate_(o, packed[:, self.gate_at:self.gate_at + self.q_size])
         y = self.o.forward(o, allow_partials=True)
         if self.out_bias_on:
+            if getattr(self, "defer_bias", False):       # the caller adds it where it adds the output itself
+                from .hybrid import Biased
+                return Biased(y, self.o_bias)
             y = ops.add_bias(y, self.o_bias, self.o.weight.dtype)
         return y

@@ -109,7 +109,11 @@ class OutputNormBlock(Part):
         else:                                # behind a layer that leaves its output to be added
             stream = residual + (h.sum(0) if h.dim() == 3 else h).float()
             x = stream.to(h.dtype if h.dim() == 2 else self.norm1.out_dtype)
-        x, stream = self.norm1.add_to(self.mixer.forward(x, step, cache, state), stream)
+        if getattr(self.mixer, "returns_terms", False) and hasattr(self.norm1, "add_terms"):
+            # a mixer that is a weighted sum of several outputs: sum, norm and residual sum as one kernel
+            x, stream = self.norm1.add_terms(self.mixer.forward(x, step, cache, state, terms=True), stream)
+        else:
+            x, stream = self.norm1.add_to(self.mixer.forward(x, step, cache, state), stream)
         if self.feed_forward is not None:
             x, stream = self.norm2.add_to(one_tensor(self.feed_forward.forward(x)), stream)
         return Settled(x), stream

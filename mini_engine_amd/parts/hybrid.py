@@ -34,7 +34,8 @@ class SideBySide(Mixer):
     With `side_stream`, in steps of few tokens the right mixer runs on a second stream beside the left one
     (`base.side_branch`)."""
 
-    side_stream = False
+    side_stream = True
+    returns_terms = True       # forward(..., terms=True) hands the two outputs on unadded
 
     def __init__(self, left: Mixer, right: Mixer, left_scale: float = 1.0, right_scale: float = 1.0):
         super().__init__()
@@ -58,6 +59,7 @@ class SideBySide(Mixer):
     def forward(self, x, step, cache, state, terms: bool = False):
         """`terms`: return the two outputs unadded (`ScaledTerms`) for a consumer that forms the weighted sum itself."""
         give = lambda i: (cache if self._cache_of == i else None, state if self._state_of == i else None)
+        self.left.defer_bias = self.right.defer_bias = True         # an output bias joins the weighted sum's kernel
         if self.side_stream and few_tokens(x):
             with side_branch(x.device, 1) as branch:
                 b = self.right.forward(x, step, *give(1))
@@ -66,8 +68,20 @@ class SideBySide(Mixer):
         else:
             a = self.left.forward(x, step, *give(0))
             b = self.right.forward(x, step, *give(1))
-        out = ScaledTerms([(a, self.left_scale, None), (b, self.right_scale, None)])
+        out = ScaledTerms([_term(a, self.left_scale), _term(b, self.right_scale)])
         return out if terms else out.value()
+
+
+class Biased:
+    """A mixer's output whose bias is still to be added: (rows or float32 partial sums, float32 bias [n]). A mixer returns
+    one only to a caller that asked for it (`defer_bias`); `SideBySide` does, and adds the bias inside its weighted sum."""
+
+    def __init__(self, rows: torch.Tensor, bias: torch.Tensor):
+        self.rows, self.bias = rows, bias
+
+
+def _term(y, scale: float) -> tuple:
+    return (y.rows, scale, y.bias) if isinstance(y, Biased) else (y, scale, None)
 
 
 def _decay_base(shape, generator, device):

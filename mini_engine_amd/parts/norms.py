@@ -47,6 +47,11 @@ class RMSNorm(Norm):
         partial sums [P, T, n]. -> (the new stream in the compute dtype, the new stream in float32)."""
         return ops.add_rms_norm(y, self.weight, self.eps, stream, self.out_dtype)
 
+    def add_terms(self, terms, stream):
+        """`add_to` on a weighted sum that has not been formed yet: `terms.terms` lists (rows or float32 partial sums,
+        scale, bias or None); sum, norm and residual sum are one kernel (`ops.weighted_sum`)."""
+        return ops.weighted_sum(terms.terms, self.weight, self.eps, stream, self.out_dtype)
+
     def forward(self, x, residual, want_residual: bool = True):
         return ops.rms_norm(x, self.weight, self.eps, residual, self.out_dtype, want_residual)
 

@@ -301,5 +301,7 @@ def test_launch_rule_of_the_recurrence():
     for N in range(1, 257):
         for P_ in (1, 16, 64, 80, 128):
             for B, H in ((1, 1), (4, 16), (64, 32)):
-                rg = ops.decay_row_groups(B, H, N, P_)
-                assert rg in (1, 4) and (rg == 4 or N <= 64)
+                rg, prepared = ops.decay_row_groups(B, H, N, P_)
+                assert not prepared and rg in (1, 4) and (rg == 4 or N <= 64)
+                rg, prepared = ops.decay_row_groups(B, H, N, P_, 700)
+                assert prepared and rg in (4, 16) and (rg == 4 or B * H * -(-P_ // 4) <= 4096)
