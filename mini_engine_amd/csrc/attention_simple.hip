@@ -153,7 +153,8 @@ extern "C" int me_attn_simple(const void* q, int64_t q_stride, void* out, int64_
 // kernel's normalised result and lse the natural logarithm of its denominator (-inf: it saw no key). With
 // (m2, l2, acc2) the kept keys' maximum, sum and weighted values, sk the sink and M the largest of lse, m2, sk:
 //   out <- (out e^(lse - M) + acc2 e^(m2 - M)) / (e^(lse - M) + l2 e^(m2 - M) + e^(sk - M)).
-// One wave per (token, head); a lane takes a key for the scores and the channels lane, lane + 64, ... for the values.
+// One wave per (token, head); for the scores four neighbouring lanes share a key, sixteen keys at a time; for the values a
+// lane takes the channels lane, lane + 64, ...
 #define AT_MAX_D 512
 template <typename T>
 __global__ void __launch_bounds__(64)
@@ -180,37 +181,42 @@ attn_tail_kernel(const T* __restrict__ q, int64_t q_stride, T* __restrict__ out,
   if (kept > 0) {
     for (int d = lane; d < D; d += 64) qs[d] = to_f32<T>(q[t * q_stride + (int64_t)h * D + d]);
     __syncthreads();
-    for (int c0 = 0; c0 < kept; c0 += 64) {
-      const int j = c0 + lane;
+    // sixteen keys at a time: four neighbouring lanes share a key, each with every fourth of the head's dimensions
+    const int part = lane & 3;
+    for (int c0 = 0; c0 < kept; c0 += 16) {
+      const int j = c0 + (lane >> 2);
       float s = -INFINITY;
-      if (j < kept) {
-        const int64_t pg = bt[j / page];
-        if (pg >= 0) {
-          const T* kr = k_cache + ((pg * Hkv + kvh) * (int64_t)page + j % page) * D;
-          float dot = 0.f;
-          for (int d = 0; d < D; ++d) dot += qs[d] * to_f32<T>(kr[d]);
-          s = dot * scale;
-          if (softcap > 0.f) s = softcap * tanhf(s / softcap);
-        }
+      int64_t pg = -1;
+      if (j < kept) pg = bt[j / page];
+      float dot = 0.f;
+      if (pg >= 0) {
+        const T* kr = k_cache + ((pg * Hkv + kvh) * (int64_t)page + j % page) * D;
+        for (int d = part; d < D; d += 4) dot += qs[d] * to_f32<T>(kr[d]);      // neighbours read neighbouring words
+      }
+      dot += __shfl_xor(dot, 1, ME_WAVE);
+      dot += __shfl_xor(dot, 2, ME_WAVE);
+      if (pg >= 0) {
+        s = dot * scale;
+        if (softcap > 0.f) s = softcap * tanhf(s / softcap);
       }
       const float m_new = fmaxf(m2, wave_max(s));
       const float p = (s > -INFINITY) ? expf(s - m_new) : 0.f;
       const float alpha = (m2 == -INFINITY) ? 0.f : expf(m2 - m_new);
-      l2 = l2 * alpha + wave_sum(p);
+      l2 = l2 * alpha + wave_sum(part == 0 ? p : 0.f);
       m2 = m_new;
       __syncthreads();
-      sc[lane] = p;
+      if (part == 0) sc[lane >> 2] = p;
       __syncthreads();
-      const int je = min(64, kept - c0);
+      const int je = min(16, kept - c0);
 #pragma unroll
       for (int i = 0; i < AT_MAX_D / 64; ++i) {
         const int d = lane + 64 * i;
         if (d < D) {
           float a = 0.f;
           for (int jj = 0; jj < je; ++jj) {
-            const int64_t pg = bt[(c0 + jj) / page];
-            if (pg < 0) continue;
-            a += sc[jj] * to_f32<T>(v_cache[((pg * Hkv + kvh) * (int64_t)D + d) * page + (c0 + jj) % page]);
+            const int64_t vp = bt[(c0 + jj) / page];
+            if (vp < 0) continue;
+            a += sc[jj] * to_f32<T>(v_cache[((vp * Hkv + kvh) * (int64_t)D + d) * page + (c0 + jj) % page]);
           }
           acc[i] = acc[i] * alpha + a;
         }
