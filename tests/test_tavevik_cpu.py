@@ -259,11 +259,8 @@ def test_the_weights_show_a_mechanism_that_is_left_out(tavevik_folders, spoil):
 
 # ---------------------------------------------------------------- the engine against the plain evaluation
 
-# every case on the configuration with both kinds; the others (more layers, each kind alone) where they differ most:
-# token by token, portions down to two tokens, and the batch with its page and slot reuse (the GPU tests run all of them)
-@pytest.mark.parametrize("case,name", [(case, "pair") for case in C.ALL]
-                         + [(C.token_by_token, "order"), (C.batch_against_alone, "order"), (C.portions, "one"), (C.portions, "two"),
-                            (C.slots_start_from_zero, "two")], ids=lambda v: getattr(v, "__name__", v))
+@pytest.mark.parametrize("name", ["pair", "order", "one", "two"])
+@pytest.mark.parametrize("case", C.ALL, ids=lambda c: c.__name__)
 def test_cuts(tavevik_folders, plain_backend, case, name):
     case(Env(tavevik_folders), name)
 
@@ -272,7 +269,7 @@ def test_far_keys_and_window_edges(tavevik_folders, plain_backend):
     C.window_edges(Env(tavevik_folders))
 
 
-@pytest.mark.parametrize("name", ["pair"])
+@pytest.mark.parametrize("name", ["pair", "order"])
 def test_greedy_generation_through_the_scheduler(tavevik_folders, plain_backend, name):
     C.greedy_through_the_engine("cpu", "float32", name, tavevik_folders(name), exact=True)
 
