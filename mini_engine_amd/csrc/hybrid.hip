@@ -398,7 +398,10 @@ __global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a, const float* _
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
           const int n = lane + 64 * i;
-          if (n < NR) { sq[buf][j][n] = nq[j][i]; sk[buf][j][n] = nk[j][i]; sd[buf][j][n] = nr[j][i]; }
+          // row n belongs to lane n % RG of a column as its row n / RG: a lane's rows lie side by side in LDS, so that it
+          // reads them four at a time
+          const int at = (n % RG) * RL + n / RG;
+          if (n < NR) { sq[buf][j][at] = nq[j][i]; sk[buf][j][at] = nk[j][i]; sd[buf][j][at] = nr[j][i]; }
         }
         cv[j] = nv[j];
         cx[j] = x;
@@ -418,7 +421,7 @@ __global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a, const float* _
         if (RULE == 0) {
 #pragma unroll
           for (int i = 0; i < RL; ++i) {
-            const int n = i * RG + rg;
+            const int n = rg * RL + i;
             y = fmaf(sq[buf][j][n], S[i], y);
             S[i] = fmaf(sd[buf][j][n], S[i], sk[buf][j][n] * v);
           }
@@ -426,7 +429,7 @@ __global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a, const float* _
           float dot = 0.f;
 #pragma unroll
           for (int i = 0; i < RL; ++i) {
-            const int n = i * RG + rg;
+            const int n = rg * RL + i;
             S[i] *= sd[buf][j][n];
             dot = fmaf(S[i], sk[buf][j][n], dot);
           }
@@ -434,7 +437,7 @@ __global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a, const float* _
           const float u = cx[j] * (v - dot);
 #pragma unroll
           for (int i = 0; i < RL; ++i) {
-            const int n = i * RG + rg;
+            const int n = rg * RL + i;
             S[i] = fmaf(sk[buf][j][n], u, S[i]);
             y = fmaf(S[i], sq[buf][j][n], y);
           }

@@ -49,6 +49,7 @@ class SideBySide(Mixer):
         self._cache_of = 0 if needs[0] is not None else (1 if needs[1] is not None else None)
         self._state_of = 0 if states[0] is not None else (1 if states[1] is not None else None)
         self.capturable = getattr(left, "capturable", True) and getattr(right, "capturable", True)
+        left.defer_bias = right.defer_bias = True         # an output bias joins the weighted sum's kernel (`Biased`)
 
     def cache_need(self):
         return None if self._cache_of is None else (self.left, self.right)[self._cache_of].cache_need()
@@ -59,7 +60,6 @@ class SideBySide(Mixer):
     def forward(self, x, step, cache, state, terms: bool = False):
         """`terms`: return the two outputs unadded (`ScaledTerms`) for a consumer that forms the weighted sum itself."""
         give = lambda i: (cache if self._cache_of == i else None, state if self._state_of == i else None)
-        self.left.defer_bias = self.right.defer_bias = True         # an output bias joins the weighted sum's kernel
         if self.side_stream and few_tokens(x):
             with side_branch(x.device, 1) as branch:
                 b = self.right.forward(x, step, *give(1))

@@ -272,3 +272,18 @@ def test_trace_program_on_this_design(tavevik_folders, tmp_path, dtype):
     for r, g in TR.collect(steps, out, V).items():
         err = helpers.rel_err(g, C.plain_logits(folder, ids[r]))
         assert err <= TOL[getattr(torch, dtype)], f"{dtype} request {r}: {err:.3g}"
+
+
+def test_offline_workload_row_with_random_weights(tmp_path, capsys):
+    """The offline workload through the command line, on this design at a tiny size with random weights."""
+    import json
+    from mini_engine_amd import cli
+    rc = cli.main(["--random-weights", "tavevik:tinyA", "--num-seqs", "6", "--max-prompt", "40", "--max-output", "8",
+                   "--max-model-len", "64", "--max-num-seqs", "4", "--budget", "32", "--tokens-out", "-",
+                   "--out", str(tmp_path / "bench.jsonl")])
+    assert rc == 0
+    lines = capsys.readouterr().out.strip().splitlines()
+    row = json.loads(lines[-1])
+    tokens = [json.loads(line) for line in lines[-7:-1]]
+    assert [len(t) for t in tokens] == [8] * 6 and all(0 <= t < 256 for ts in tokens for t in ts)
+    assert row["num_seqs"] == 6 and row["output_tokens"] == 48 and row["throughput_tok_s"] > 0
