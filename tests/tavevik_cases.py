@@ -68,6 +68,12 @@ CONFIGS = {
     # each kind alone; a convolution of one tap (no inputs to carry)
     "one": _model(64, 32, 1e-6, [_one(_left(6, 2, 16, 16, 0.25, 8, 1e4, 6, keep=2, cap=3.0), 4, 8, 8, ff=48)]),
     "two": _model(64, 32, 1e-5, [_two(_left(3, 1, 16, 32, 0.25, 16, 1e4, 5), 2, 2, 8, 16, 1, 8, 8, ff=40)]),
+    # sizes in no whole steps of 8: a width of 36, thin pairs of 12 and 20, head sizes of 40 and 24, an odd vocabulary, five
+    # heads on one key head, a state of 96 x 20
+    "odd": _model(131, 36, 1e-5, [
+        _two(_left(5, 1, 40, 24, 0.16, 10, 1234.5, 19), 3, 1, 96, 20, 3, 12, 20, ff=52),
+        _one(_left(2, 1, 24, 40, 0.2, 24, 9e4, 4, keep=9), 3, 20, 12, ff=44, limit=3.0),
+    ]),
     # windows of hundreds of positions: keys far back; states of 72 and 80 rows (four lanes to a column), values of 80
     "far": _model(80, 32, 1e-5, [
         _one(_left(3, 1, 32, 16, 0.2, 32, 4e5, 300, keep=4, cap=20.0), 1, 72, 8, ff=40),
@@ -79,8 +85,8 @@ CONFIGS["real"] = _model(1000, 512, 1e-6, [
     _two(_left(8, 2, 128, 128, 128 ** -0.5, 64, 1e6, 256), 4, 2, 128, 128, 4, 32, 32, ff=1024, limit=7.0),
     _one(_left(8, 4, 64, 64, 0.125, 64, 1e6, 128, keep=16, cap=50.0), 8, 64, 32, ff=1024, limit=7.0),
 ])
-SEEDS = {"pair": 21, "order": 22, "one": 23, "two": 24, "far": 25, "real": 26}
-PAGE = {"pair": 8, "order": 16, "one": 16, "two": 8, "far": 16, "real": 16}
+SEEDS = {"pair": 21, "order": 22, "one": 23, "two": 24, "far": 25, "real": 26, "odd": 27}
+PAGE = {"pair": 8, "order": 16, "one": 16, "two": 8, "far": 16, "real": 16, "odd": 8}
 SHARPEN = 3.0
 
 

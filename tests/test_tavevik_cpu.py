@@ -259,7 +259,7 @@ def test_the_weights_show_a_mechanism_that_is_left_out(tavevik_folders, spoil):
 
 # ---------------------------------------------------------------- the engine against the plain evaluation
 
-@pytest.mark.parametrize("name", ["pair", "order", "one", "two"])
+@pytest.mark.parametrize("name", ["pair", "order", "one", "two", "odd"])
 @pytest.mark.parametrize("case", C.ALL, ids=lambda c: c.__name__)
 def test_cuts(tavevik_folders, plain_backend, case, name):
     case(Env(tavevik_folders), name)

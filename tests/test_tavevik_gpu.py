@@ -18,6 +18,12 @@ DEV = "cuda"
 TOL = {torch.float32: 5e-5, torch.bfloat16: 1.2e-1}    # widths of 32-48 make bfloat16 noisy: the plain twins in bfloat16 differ as much (to the digit)
 
 
+# The configuration of odd sizes (width 36) is ill-conditioned in bfloat16 at single positions: with the attention kernel swapped
+# for the exact one, every attention output equal within one rounding (0.002), the logits of one position of 50 move by 0.14.
+# Its bfloat16 runs are held to a loose bound; its float32 runs to the same one as every other configuration.
+LOOSE_BF16 = {"odd": 2.5e-1}
+
+
 def hip():
     return ops.HipBackend()
 
@@ -199,6 +205,7 @@ class Env:
 
     def runner(self, name, pages, slots):
         folder = self.folders(name)
+        self.tol = LOOSE_BF16.get(name, TOL[self.dtype]) if self.dtype == torch.bfloat16 else TOL[self.dtype]
         if name not in self.models:
             self.models[name] = load_model(folder, self.device, self.dtype, 1024)
         model = self.models[name]
@@ -212,7 +219,7 @@ def env(request, tavevik_folders):
     return Env(tavevik_folders, request.param)
 
 
-@pytest.mark.parametrize("name", ["pair", "order", "one", "two"])
+@pytest.mark.parametrize("name", ["pair", "order", "one", "two", "odd"])
 @pytest.mark.parametrize("case", C.ALL, ids=lambda c: c.__name__)
 def test_cuts(env, case, name):
     case(env, name)
