@@ -661,3 +661,230 @@ class TavevikConfig:
     def flat(self) -> dict[str, Any]:
         return {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "num_hidden_layers": len(self.layers),
                 "layer_kinds": [layer.kind for layer in self.layers]}
+
+
+# ------------------------------------------------------------------------------------ Goluzen
+@dataclass(frozen=True)
+class GoluzenLayer:
+    """One entry of a Goluzen config's `layers`: which mixer it has, the mixer's sizes and constants with the optional
+    keys resolved, and the feed-forward's (None: the layer has no feed-forward)."""
+
+    kind: str                  # "attention", "latent_attention" or "gla"
+    mixer: dict
+    mlp: dict | None
+
+
+def _scaling(rot: dict | None, kind: str, where: str) -> dict | None:
+    """`rot.scaling` as the rotary encoding takes it: {"kind": "linear" | "yarn", ...} or None."""
+    sc = rot.get("scaling") if rot else None
+    if not sc:
+        return None
+    out = {"kind": kind, "factor": _need(sc, "factor", float, where)}
+    if kind == "yarn":
+        out["original"] = _need(sc, "original", float, where)
+        out["fast"] = _need(sc, "fast", float, where)
+        out["slow"] = _need(sc, "slow", float, where)
+    return out
+
+
+@register_config("Goluzen")
+@dataclass(frozen=True)
+class GoluzenConfig:
+    """The ``config.json`` keys of the Goluzen design: pre-norm layers (norm weights stored around zero) that each name
+    their mixer. `attention`: grouped heads with biases on q, k and v, a rotation of the first dimensions of each head
+    (pairs half the rotating width apart) whose rates are divided by a factor, q and k at unit root mean square, scores
+    bent under a cap, a trailing window that keeps the first positions visible, a sink per head. `latent_attention`:
+    keys and values made head by head from a cached latent and one shared rotated key part (adjacent pairs, YaRN
+    scaling), a trailing window, a gate on the heads' outputs; with `kv_from` the latent of an earlier layer. `gla`:
+    linear attention with a decay per key channel from a thin matrix pair (`decay_rank` comes from the checkpoint's
+    tensors when the file does not name it). Feed-forwards: dense with the tanh form of gelu, or routed experts without
+    gates (sigmoid scores, a correction for the choice, groups scored by their two best, weights times a constant)
+    beside an optional shared expert under a gate per token. The embedding's rows are multiplied by `embedding.scale`;
+    the head has weights of its own. Every size and constant comes from the file."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    embedding_scale: float
+    layers: tuple
+    eos_token_id: int | None = None
+    max_position_embeddings: int | None = None
+
+    KINDS = ("attention", "latent_attention", "gla")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, raw: dict[str, Any]) -> "GoluzenConfig":
+        norm = raw.get("norm")
+        if not isinstance(norm, dict):
+            raise ConfigError("config.json lacks the object 'norm'")
+        listed = raw.get("layers")
+        if not isinstance(listed, list) or not listed:
+            raise ConfigError("config.json lacks the list 'layers'")
+        layers = []
+        for i, entry in enumerate(listed):
+            where = f"layers[{i}]"
+            kind = entry.get("type") if isinstance(entry, dict) else None
+            if kind not in cls.KINDS:
+                raise ConfigError(f"{where}: 'type' must be one of {list(cls.KINDS)}, got {kind!r}")
+            m = entry.get("mixer")
+            if not isinstance(m, dict):
+                raise ConfigError(f"{where} lacks the object 'mixer'")
+            at = where + ".mixer"
+            rot, mask = m.get("rot"), m.get("mask")
+            if kind == "attention":
+                mixer = {key: _need(m, key, typ, at) for key, typ in (("heads", int), ("dim", int), ("vdim", int), ("scale", float))}
+                mixer["kv_heads"] = _need(m, "kv_heads", int, at) if m.get("kv_heads") is not None else mixer["heads"]
+                mixer["rot_dims"] = _need(rot, "dims", int, at + ".rot") if rot else 0
+                mixer["rot_base"] = _need(rot, "base", float, at + ".rot") if rot else 1.0
+                mixer["rot_scaling"] = _scaling(rot, "linear", at + ".rot.scaling")
+                mixer["window"] = _need(mask, "size", int, at + ".mask") if mask else None
+                mixer["keep_first"] = int(mask.get("keep_first") or 0) if mask else 0
+                mixer["softcap"] = float(m["softcap"]) if m.get("softcap") else None
+            elif kind == "latent_attention":
+                mixer = {key: _need(m, key, typ, at) for key, typ in (("heads", int), ("dim", int), ("rot_dim", int), ("vdim", int),
+                                                                       ("kv_rank", int), ("scale", float))}
+                mixer["rot_base"] = _need(rot, "base", float, at + ".rot") if rot else 1.0
+                if rot and rot.get("dims") is not None and int(rot["dims"]) != mixer["rot_dim"]:
+                    raise ConfigError(f"{at}: rot.dims must equal rot_dim")
+                mixer["rot_scaling"] = _scaling(rot, "yarn", at + ".rot.scaling")
+                mixer["window"] = _need(mask, "size", int, at + ".mask") if mask else None
+                mixer["kv_from"] = _need(m, "kv_from", int, at) if m.get("kv_from") is not None else None
+            else:
+                mixer = {key: _need(m, key, typ, at) for key, typ in (("heads", int), ("dim", int), ("vdim", int), ("tau", float))}
+                mixer["decay_rank"] = m.get("decay_rank")
+            mlp = entry.get("mlp")
+            ff = None
+            if mlp is not None:
+                fkind = mlp.get("kind")
+                if fkind == "dense":
+                    ff = {"kind": "dense", "ff": _need(mlp, "ff", int, where + ".mlp")}
+                elif fkind == "moe":
+                    router = mlp.get("router")
+                    if not isinstance(router, dict) or not isinstance(mlp.get("expert"), dict):
+                        raise ConfigError(f"{where}.mlp lacks the objects 'router' and 'expert'")
+                    groups, shared = router.get("groups"), mlp.get("shared")
+                    ff = {"kind": "moe", "ff": _need(mlp["expert"], "ff", int, where + ".mlp.expert"),
+                          "experts": _need(router, "experts", int, where + ".mlp.router"),
+                          "top": _need(router, "top", int, where + ".mlp.router"),
+                          "scale": float(router["scale"]) if router.get("scale") is not None else 1.0,
+                          "group_count": _need(groups, "count", int, where + ".mlp.router.groups") if groups else 1,
+                          "group_keep": _need(groups, "keep", int, where + ".mlp.router.groups") if groups else 1,
+                          "shared_ff": _need(shared, "ff", int, where + ".mlp.shared") if shared else None}
+                else:
+                    raise ConfigError(f"{where}.mlp: 'kind' must be 'dense' or 'moe', got {fkind!r}")
+            layers.append(GoluzenLayer(kind, mixer, ff))
+        emb = raw.get("embedding") or {}
+        cfg = cls(vocab_size=_need(raw, "vocab", int), hidden_size=_need(raw, "width", int),
+                  norm_eps=_need(norm, "eps", float, "config.json norm"),
+                  embedding_scale=float(emb["scale"]) if emb.get("scale") is not None else 1.0, layers=tuple(layers),
+                  eos_token_id=raw.get("eos_token_id"), max_position_embeddings=raw.get("max_position_embeddings"))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.vocab_size < 1 or self.hidden_size < 1 or not self.norm_eps > 0:
+            raise ConfigError("vocab and width must be positive and norm.eps above zero")
+        for i, layer in enumerate(self.layers):
+            m, where = layer.mixer, f"layers[{i}]"
+            if any(v < 1 for k, v in m.items() if k in ("heads", "kv_heads", "dim", "vdim", "kv_rank")) or not m.get("scale", 1.0) > 0:
+                raise ConfigError(f"{where}: sizes and the score scale must be positive")
+            if m.get("window") is not None and m["window"] < 1:
+                raise ConfigError(f"{where}: mask.size must be positive")
+            if layer.kind == "attention":
+                if m["heads"] % m["kv_heads"]:
+                    raise ConfigError(f"{where}: {m['heads']} heads are not a multiple of {m['kv_heads']} kv_heads")
+                if m["rot_dims"] % 2 or not 0 <= m["rot_dims"] <= m["dim"]:
+                    raise ConfigError(f"{where}: rot.dims must be even and at most dim")
+                if m["keep_first"] < 0 or (m["keep_first"] and m["window"] is None):
+                    raise ConfigError(f"{where}: mask.keep_first needs mask.size and must not be negative")
+                if m["softcap"] is not None and not m["softcap"] > 0:
+                    raise ConfigError(f"{where}: softcap must be positive")
+            elif layer.kind == "latent_attention":
+                if m["rot_dim"] < 0 or m["rot_dim"] % 2:
+                    raise ConfigError(f"{where}: rot_dim must be even")
+                src = m["kv_from"]
+                if src is not None:
+                    if not 0 <= src < i or self.layers[src].kind != "latent_attention" or self.layers[src].mixer["kv_from"] is not None:
+                        raise ConfigError(f"{where}: kv_from must name an earlier latent_attention layer that makes its own latent")
+                    theirs = self.layers[src].mixer
+                    if any(theirs[k] != m[k] for k in ("kv_rank", "rot_dim", "rot_base", "rot_scaling")):
+                        raise ConfigError(f"{where}: the layer named by kv_from has another latent size or rotation")
+            else:
+                if not m["tau"] > 0 or (m["decay_rank"] is not None and int(m["decay_rank"]) < 1):
+                    raise ConfigError(f"{where}: tau and decay_rank must be positive")
+            for sc in (m.get("rot_scaling"),):
+                if sc is not None and (not sc["factor"] > 0 or (sc["kind"] == "yarn" and not (sc["original"] > 0 and sc["fast"] > 0 and sc["slow"] > 0))):
+                    raise ConfigError(f"{where}: rot.scaling's numbers must be positive")
+            f = layer.mlp
+            if f is not None and f["ff"] < 1:
+                raise ConfigError(f"{where}.mlp: ff must be positive")
+            if f is not None and f["kind"] == "moe":
+                if f["experts"] < 1 or not 1 <= f["top"] <= f["experts"]:
+                    raise ConfigError(f"{where}.mlp: experts must be positive and top at most experts")
+                if f["group_count"] < 1 or f["experts"] % f["group_count"] or not 1 <= f["group_keep"] <= f["group_count"]:
+                    raise ConfigError(f"{where}.mlp: {f['experts']} experts do not form {f['group_count']} equal groups "
+                                      f"of which {f['group_keep']} are kept")
+                if f["group_keep"] * (f["experts"] // f["group_count"]) < f["top"]:
+                    raise ConfigError(f"{where}.mlp: the kept groups hold fewer experts than a token uses")
+                if f["shared_ff"] is not None and f["shared_ff"] < 1:
+                    raise ConfigError(f"{where}.mlp.shared: ff must be positive")
+
+    def to_dict(self) -> dict[str, Any]:
+        """A ``config.json`` that reads back to an equal config."""
+        def scaling(sc):
+            return {k: v for k, v in sc.items() if k != "kind"}
+
+        out = []
+        for layer in self.layers:
+            x = layer.mixer
+            if layer.kind == "attention":
+                m = {k: x[k] for k in ("heads", "kv_heads", "dim", "vdim", "scale")}
+                if x["rot_dims"]:
+                    m["rot"] = {"dims": x["rot_dims"], "base": x["rot_base"]}
+                    if x["rot_scaling"]:
+                        m["rot"]["scaling"] = scaling(x["rot_scaling"])
+                if x["window"] is not None:
+                    m["mask"] = {"size": x["window"]}
+                    if x["keep_first"]:
+                        m["mask"]["keep_first"] = x["keep_first"]
+                if x["softcap"] is not None:
+                    m["softcap"] = x["softcap"]
+            elif layer.kind == "latent_attention":
+                m = {k: x[k] for k in ("heads", "dim", "rot_dim", "vdim", "kv_rank", "scale")}
+                m["rot"] = {"dims": x["rot_dim"], "base": x["rot_base"]}
+                if x["rot_scaling"]:
+                    m["rot"]["scaling"] = scaling(x["rot_scaling"])
+                if x["window"] is not None:
+                    m["mask"] = {"size": x["window"]}
+                if x["kv_from"] is not None:
+                    m["kv_from"] = x["kv_from"]
+            else:
+                m = {k: x[k] for k in ("heads", "dim", "vdim", "tau")}
+                if x["decay_rank"] is not None:
+                    m["decay_rank"] = x["decay_rank"]
+            f = layer.mlp
+            mlp = None
+            if f is not None and f["kind"] == "dense":
+                mlp = {"kind": "dense", "ff": f["ff"]}
+            elif f is not None:
+                mlp = {"kind": "moe", "expert": {"ff": f["ff"]},
+                       "router": {"experts": f["experts"], "top": f["top"], "scale": f["scale"],
+                                  "groups": {"count": f["group_count"], "keep": f["group_keep"]}}}
+                if f["shared_ff"] is not None:
+                    mlp["shared"] = {"ff": f["shared_ff"]}
+            out.append({"type": layer.kind, "mixer": m, "mlp": mlp})
+        d = {"architecture": self.architecture_name, "vocab": self.vocab_size, "width": self.hidden_size,
+             "norm": {"eps": self.norm_eps}, "embedding": {"scale": self.embedding_scale}, "layers": out}
+        if self.eos_token_id is not None:
+            d["eos_token_id"] = self.eos_token_id
+        if self.max_position_embeddings is not None:
+            d["max_position_embeddings"] = self.max_position_embeddings
+        return d
+
+    def flat(self) -> dict[str, Any]:
+        return {"vocab_size": self.vocab_size, "hidden_size": self.hidden_size, "num_hidden_layers": len(self.layers),
+                "layer_kinds": [layer.kind for layer in self.layers]}

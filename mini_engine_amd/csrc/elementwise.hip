@@ -44,6 +44,29 @@ extern "C" int me_gather_rows(const void* src, const int32_t* idx, void* out, in
   return 0;
 }
 
+// out[r, :] = scale * src[idx[r], :] in float32: embedding rows under a multiplier start the 32-bit stream unrounded.
+template <typename TX>
+__global__ void gather_rows_scaled_kernel(const TX* __restrict__ src, const int32_t* __restrict__ idx, float* __restrict__ out,
+                                          int64_t n, int64_t num_src_rows, float scale) {
+  const int64_t r = blockIdx.x;
+  int64_t s = idx[r];
+  if (s < 0 || s >= num_src_rows) s = 0;
+  for (int64_t i = threadIdx.x; i < n; i += blockDim.x) out[r * n + i] = scale * to_f32<TX>(src[s * n + i]);
+}
+
+extern "C" int me_gather_rows_scaled(const void* src, int dtype, const int32_t* idx, float* out, int64_t num_rows, int64_t n,
+                                     int64_t num_src_rows, float scale, hipStream_t stream) {
+  if (num_rows == 0) return 0;
+  ME_CHECK(n > 0 && num_src_rows > 0, "gather_rows_scaled: empty source");
+  const int threads = n >= 1024 ? 256 : (n > 256 ? 128 : 64);
+  if (dtype == ME_F32)
+    gather_rows_scaled_kernel<float><<<dim3(num_rows), dim3(threads), 0, stream>>>((const float*)src, idx, out, n, num_src_rows, scale);
+  else
+    gather_rows_scaled_kernel<bf16_t><<<dim3(num_rows), dim3(threads), 0, stream>>>((const bf16_t*)src, idx, out, n, num_src_rows, scale);
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
 // ------------------------------------------------------------------ tokens handed over on the device
 // tokens[r] = sampled[take[r]] for the rows whose take[r] >= 0; the other rows keep what they hold. A decode step
 // that is launched before the step in flight has delivered its tokens takes them so from the sampling kernel's

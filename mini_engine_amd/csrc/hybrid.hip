@@ -89,13 +89,15 @@ extern "C" int me_glu_clamped(const void* gu, int64_t gu_stride, void* out, int 
 }
 
 // ------------------------------------------------------------------ weighted sum of sublayer outputs
-// out[t, c] = sum_i scale_i * ((sum_p term_i[p, t, c]) + bias_i[c]), float32. Terms are rows in the compute dtype or
-// stacked float32 partial sums. With w: the norm on the sum as well, stream' = stream + w * out / rms(out), one
+// out[t, c] = sum_i scale_i * gate_i[t] * ((sum_p term_i[p, t, c]) + bias_i[c]), float32. Terms are rows in the compute dtype or
+// stacked float32 partial sums. gate_i[t] = sigmoid(g_i[t * gate_stride_i]) for a term that has gate rows g_i (in the compute
+// dtype or float32), else 1. With w: the norm on the sum as well, stream' = stream + w * out / rms(out), one
 // workgroup per row (the sum is held in LDS between the two passes), the new stream also rounded to TY.
 #define WS_MAX_TERMS 4
 struct WsArgs {
   const void* term[WS_MAX_TERMS]; int dtype[WS_MAX_TERMS]; int parts[WS_MAX_TERMS]; int64_t part_stride[WS_MAX_TERMS];
   float scale[WS_MAX_TERMS]; const float* bias[WS_MAX_TERMS];
+  const void* gate[WS_MAX_TERMS]; int gate_dtype[WS_MAX_TERMS]; int64_t gate_stride[WS_MAX_TERMS];
   int count, n;
 };
 
@@ -110,6 +112,11 @@ __device__ __forceinline__ float ws_value(const WsArgs& a, int64_t t, int c) {
       v = to_f32<bf16_t>(((const bf16_t*)a.term[i])[t * a.n + c]);
     }
     if (a.bias[i] != nullptr) v += a.bias[i][c];
+    if (a.gate[i] != nullptr) {
+      const float g = a.gate_dtype[i] == ME_F32 ? ((const float*)a.gate[i])[t * a.gate_stride[i]]
+                                                : to_f32<bf16_t>(((const bf16_t*)a.gate[i])[t * a.gate_stride[i]]);
+      v *= 1.0f / (1.0f + expf(-g));
+    }
     total += a.scale[i] * v;
   }
   return total;
@@ -147,7 +154,7 @@ __global__ void weighted_sum_norm_kernel(WsArgs a, const float* __restrict__ w, 
 extern "C" int me_weighted_sum(int count, const void** terms, const int* dtypes, const int* parts, const int64_t* part_strides,
                                const float* scales, const float** biases, float* out, const float* w, float eps,
                                const float* stream_in, float* stream_out, void* rounded, int rounded_dtype, int64_t T, int n,
-                               hipStream_t stream) {
+                               const void** gates, const int* gate_dtypes, const int64_t* gate_strides, hipStream_t stream) {
   if (T == 0 || n == 0) return 0;
   ME_CHECK(count >= 1 && count <= WS_MAX_TERMS, "weighted_sum: 1..%d terms", WS_MAX_TERMS);
   WsArgs a;
@@ -156,6 +163,7 @@ extern "C" int me_weighted_sum(int count, const void** terms, const int* dtypes,
     ME_CHECK(parts[i] >= 1 && (dtypes[i] == ME_F32 || parts[i] == 1), "weighted_sum: partial sums are float32");
     a.term[i] = terms[i]; a.dtype[i] = dtypes[i]; a.parts[i] = parts[i]; a.part_stride[i] = part_strides[i];
     a.scale[i] = scales[i]; a.bias[i] = biases[i];
+    a.gate[i] = gates ? gates[i] : nullptr; a.gate_dtype[i] = gates ? gate_dtypes[i] : ME_F32; a.gate_stride[i] = gates ? gate_strides[i] : 0;
   }
   if (w == nullptr) {
     const int64_t total = T * n;
@@ -225,6 +233,8 @@ extern "C" int me_token_shift(const void* x, int64_t x_stride, int dtype, const 
 //   RULE 1 (delta):  d_n = exp(-rate[h] softplus(raw[t, h, n] + base[h, n])),  beta = sigmoid(beta_raw[t, h]);
 //                    S[n, p] <- d_n S[n, p];  u_p = beta (v_p - sum_n S[n, p] k_n);  S[n, p] <- S[n, p] + k_n u_p;
 //                    y_p = sum_n S[n, p] q_n
+//   RULE 2 (gated):  d_n = sigmoid(raw[t, h, n] + base[h, n]) ^ rate[h] = exp(-rate[h] softplus(-(raw + base)));
+//                    S[n, p] <- d_n S[n, p] + k_n v_p;   y_p = sum_n S[n, p] q_n
 // With `unit`: q and k are first divided by sqrt(sum of their squares + unit_eps) per head; q is multiplied by q_scale.
 // Every sum runs over n only, so a column p of the state never meets another: a wave takes 64 / RG columns of one head
 // and a lane NR / RG of a column's rows, kept in registers for the whole walk; with RG > 1 the RG lanes of a column,
@@ -283,10 +293,12 @@ __device__ __forceinline__ float shape_token(const DrArgs& a, int lane, int nr_r
     k[i] *= ks;
     float dv;
     if (RULE == 0) dv = expf(-expf(d[i] + base[i]));
+    else if (RULE == 2) dv = expf(-rate * hy_softplus(-(d[i] + base[i])));
     else dv = expf(-rate * hy_softplus(d[i] + base[i]));
     d[i] = (n < a.N && n < nr_rows) ? dv : 1.0f;
     own += q[i] * bonus[i] * k[i];
   }
+  if (RULE == 2) return 0.f;
   return RULE == 1 ? hy_sigmoid(beta) : wave_sum(own);
 }
 
@@ -312,7 +324,7 @@ __global__ void __launch_bounds__(64) decay_prepare_kernel(DrArgs a, float* __re
     d[i] = in ? to_f32<TX>(rp[t * a.raw_stride + h * a.N + n]) : 0.f;
   }
   const float beta = RULE == 1 ? to_f32<TX>(bp[t * a.beta_stride + h]) : 0.f;
-  const float x = shape_token<PER, RULE>(a, lane, NR, q, k, d, base, bonus, RULE == 1 ? a.rate[h] : 0.f, beta);
+  const float x = shape_token<PER, RULE>(a, lane, NR, q, k, d, base, bonus, RULE != 0 ? a.rate[h] : 0.f, beta);
   const int64_t at = (t * a.H + h) * NR;
 #pragma unroll
   for (int i = 0; i < PER; ++i) {
@@ -359,7 +371,7 @@ __global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a, const float* _
     base[i] = in ? a.base[h * a.N + n] : 0.f;
     bonus[i] = (RULE == 0 && in) ? a.bonus[h * a.N + n] : 0.f;
   }
-  const float rate = (RULE == 1 && !PRE) ? a.rate[h] : 0.f;
+  const float rate = (RULE != 0 && !PRE) ? a.rate[h] : 0.f;
   // a batch of tokens on its way (n*) and the batch being worked on (c*): a lane's own column's v and the token's own
   // number (the write strength, or under the bonus rule sum_n q_n bonus_n k_n)
   float nq[DR_TB][PER], nk[DR_TB][PER], nr[DR_TB][PER], nv[DR_TB], nb[DR_TB];
@@ -425,6 +437,13 @@ __global__ void __launch_bounds__(64) decay_rows_kernel(DrArgs a, const float* _
             y = fmaf(sq[buf][j][n], S[i], y);
             S[i] = fmaf(sd[buf][j][n], S[i], sk[buf][j][n] * v);
           }
+        } else if (RULE == 2) {
+#pragma unroll
+          for (int i = 0; i < RL; ++i) {
+            const int n = rg * RL + i;
+            S[i] = fmaf(sd[buf][j][n], S[i], sk[buf][j][n] * v);
+            y = fmaf(sq[buf][j][n], S[i], y);
+          }
         } else {
           float dot = 0.f;
 #pragma unroll
@@ -465,9 +484,11 @@ static void launch_decay_rows(const DrArgs& a, int rule, int num_seqs, int64_t T
     pk = pre + each; pd = pre + 2 * each; px = pre + 3 * each;
     const dim3 pgrid((unsigned)T, a.H);
     if (rule == 0) decay_prepare_kernel<TX, NR, 0><<<pgrid, block, 0, stream>>>(a, pq, pk, pd, px);
+    else if (rule == 2) decay_prepare_kernel<TX, NR, 2><<<pgrid, block, 0, stream>>>(a, pq, pk, pd, px);
     else decay_prepare_kernel<TX, NR, 1><<<pgrid, block, 0, stream>>>(a, pq, pk, pd, px);
   }
   if (rule == 0) decay_rows_kernel<TX, NR, RG, 0, PRE><<<grid, block, 0, stream>>>(a, pq, pk, pd, px);
+  else if (rule == 2) decay_rows_kernel<TX, NR, RG, 2, PRE><<<grid, block, 0, stream>>>(a, pq, pk, pd, px);
   else decay_rows_kernel<TX, NR, RG, 1, PRE><<<grid, block, 0, stream>>>(a, pq, pk, pd, px);
 }
 
@@ -482,8 +503,8 @@ extern "C" int me_decay_rows_recurrence(const void* q, int64_t q_stride, const v
   if (num_seqs == 0) return 0;
   ME_CHECK(H >= 1 && G >= 1 && H % G == 0 && N >= 1 && N <= 256 && P >= 1, "decay_rows_recurrence: %d heads over %d groups, state %d x %d "
            "(up to 256 rows)", H, G, N, P);
-  ME_CHECK(rule == 0 || rule == 1, "decay_rows_recurrence: unknown rule %d", rule);
-  ME_CHECK(rule == 0 ? bonus != nullptr : (rate != nullptr && beta != nullptr), "decay_rows_recurrence: the rule's constants are missing");
+  ME_CHECK(rule >= 0 && rule <= 2, "decay_rows_recurrence: unknown rule %d", rule);
+  ME_CHECK(rule == 0 ? bonus != nullptr : (rate != nullptr && (rule == 2 || beta != nullptr)), "decay_rows_recurrence: the rule's constants are missing");
   ME_CHECK(pre == nullptr ? (row_groups == 1 || row_groups == 4) : (row_groups == 4 || row_groups == 16),
            "decay_rows_recurrence: 1 or 4 lanes to a column, 4 or 16 over prepared values");
   ME_CHECK(T >= 0 && T <= 2147483647ll && H <= 65535, "decay_rows_recurrence: too many tokens or heads");

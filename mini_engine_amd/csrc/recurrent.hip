@@ -154,6 +154,7 @@ __global__ void activation_kernel(const TX* __restrict__ x, int64_t x_stride, TX
     float r;
     if (KIND == 0) r = silu_f(v);
     else if (KIND == 2) r = tanhf(v);
+    else if (KIND == 3) r = 0.5f * v * (1.0f + tanhf(0.7978845608028654f * (v + 0.044715f * v * v * v)));     // gelu, tanh form
     else { const float p = fmaxf(v, 0.f); r = p * p; }
     out[i] = from_f32<TX>(r);
   }
@@ -161,12 +162,12 @@ __global__ void activation_kernel(const TX* __restrict__ x, int64_t x_stride, TX
 
 extern "C" int me_activation(const void* x, int64_t x_stride, void* out, int dtype, int kind, int64_t T, int n, hipStream_t stream) {
   if (T == 0 || n == 0) return 0;
-  ME_CHECK(kind >= 0 && kind <= 2, "activation: unknown kind %d", kind);
+  ME_CHECK(kind >= 0 && kind <= 3, "activation: unknown kind %d", kind);
   const int64_t total = T * n;
   const dim3 grid((unsigned)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535)), block(256);
 #define ACT(TX, K) activation_kernel<TX, K><<<grid, block, 0, stream>>>((const TX*)x, x_stride, (TX*)out, T, n)
-  if (dtype == ME_F32) { if (kind == 0) ACT(float, 0); else if (kind == 1) ACT(float, 1); else ACT(float, 2); }
-  else { if (kind == 0) ACT(bf16_t, 0); else if (kind == 1) ACT(bf16_t, 1); else ACT(bf16_t, 2); }
+  if (dtype == ME_F32) { if (kind == 0) ACT(float, 0); else if (kind == 1) ACT(float, 1); else if (kind == 2) ACT(float, 2); else ACT(float, 3); }
+  else { if (kind == 0) ACT(bf16_t, 0); else if (kind == 1) ACT(bf16_t, 1); else if (kind == 2) ACT(bf16_t, 2); else ACT(bf16_t, 3); }
 #undef ACT
   ME_LAUNCH_CHECK();
   return 0;

@@ -29,7 +29,7 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument", "-Wno-unknown-attributes",
 ]
 CORE_SOURCES = ["elementwise.hip", "rope_kv.hip", "attention_simple.hip",
-                "gemm.hip", "gemm_mid.hip", "gemm_library.hip", "sampling.hip", "recurrent.hip", "parallel.hip", "moe.hip", "hybrid.hip"]
+                "gemm.hip", "gemm_mid.hip", "gemm_library.hip", "sampling.hip", "recurrent.hip", "parallel.hip", "moe.hip", "hybrid.hip", "latent.hip"]
 ATTN_SOURCE = "attention_mfma.hip"
 HEADERS = ["common.h", "errors.inc", "sampling.h"]
 # Head sizes that build_all() compiles ahead of use; any other multiple of 16 up to 512 is compiled when a model first needs it.

@@ -19,9 +19,9 @@ import torch
 from . import build
 
 ME_BF16, ME_F32 = 0, 1
-ACTIVATIONS = {"silu": 0, "relu2": 1, "tanh": 2}          # elementwise activations of `activation`
+ACTIVATIONS = {"silu": 0, "relu2": 1, "tanh": 2, "gelu_tanh": 3}          # elementwise activations of `activation`
 GATED_NORMS = {"silu_before": 0, "sigmoid_behind": 1, "silu_behind": 2}
-DECAY_RULES = {"bonus": 0, "delta": 1}         # update rules of `decay_rows_recurrence`
+DECAY_RULES = {"bonus": 0, "delta": 1, "gated": 2}         # update rules of `decay_rows_recurrence`
 _DT = {torch.bfloat16: ME_BF16, torch.float32: ME_F32}
 
 
@@ -59,6 +59,7 @@ class _Lib:
 P, I, L, F = c_void_p, c_int, c_int64, c_float
 _CORE_PROTOS = {
     "me_gather_rows": [P, P, P, L, L, L, P],
+    "me_gather_rows_scaled": [P, I, P, P, L, L, L, F, P],
     "me_take_tokens": [P, P, P, I, I, P],
     "me_rms_norm": [P, I, I, L, P, P, P, P, I, L, I, F, P],
     "me_silu_and_mul": [P, P, I, L, I, P],
@@ -82,15 +83,17 @@ _CORE_PROTOS = {
     "me_scaled_sum_norm": [P, I, I, P, P, P, P, P, F, P, P, P, P, P, I, L, I, F, P],
     "me_softcap": [P, L, L, I, F, P],
     "me_qkv_prepare": [P, L, P, P, P, F, I, I, F, I, P, P, P, P, P, L, I, L, I, I, I, I, I, I, P, P, L, P],
-    "me_moe_route": [P, L, I, P, L, I, I, I, I, I, P, P, P, I, P],
-    "me_moe_sort": [P, L, I, I, I, P, P, P, P, P, P, I, I, I, P],
-    "me_moe_gate_up": [P, L, P, P, P, P, P, P, L, I, I, I, I, I, P],
+    "me_moe_route": [P, L, I, P, L, I, I, I, I, I, P, P, P, I, I, I, I, F, P, P],
+    "me_moe_sort": [P, L, I, I, I, P, P, P, P, P, P, I, I, I, I, I, I, F, P, P],
+    "me_moe_gate_up": [P, L, P, P, P, P, P, P, L, I, I, I, I, I, I, P],
     "me_moe_down": [P, P, P, P, P, P, P, P, L, I, I, I, I, I, P],
-    "me_moe_experts_simple": [P, L, I, P, P, P, P, P, P, L, I, I, I, I, P],
+    "me_moe_experts_simple": [P, L, I, P, P, P, P, P, P, L, I, I, I, I, I, P],
     "me_add_bias": [P, I, I, L, L, P, I, P, I, L, I, P],
     "me_sigmoid_gate": [P, L, P, L, I, L, I, P],
     "me_glu_clamped": [P, L, P, I, L, I, F, F, P],
-    "me_weighted_sum": [I, P, P, P, P, P, P, P, P, F, P, P, P, I, L, I, P],
+    "me_weighted_sum": [I, P, P, P, P, P, P, P, P, F, P, P, P, I, L, I, P, P, P, P],
+    "me_latent_prepare": [P, L, I, I, I, I, I, I, I, I, P, F, P, L, P, P, P, L, P, P, I, L, P],
+    "me_heads_linear": [P, L, L, P, P, L, L, I, L, I, I, I, P],
     "me_token_shift": [P, L, I, P, I, P, L, P, P, P, P, L, I, P],
     "me_decay_rows_recurrence": [P, L, P, L, P, L, P, L, P, L, I, P, P, P, P, L, P, P, P, I, I, I, I, I, I, I, F, F, I, L, P, P],
     "me_sample": [P, L, P, P, P, P, I, I, P],
@@ -241,17 +244,43 @@ def library_product(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, sp
     return y
 
 
+class RouteRule:
+    """How a router's float32 logits become a choice of experts and their weights (`moe_route`). scoring: "softmax" over
+    all experts or "sigmoid" per expert; correction: float32 [experts] added to the scores for the choice only, or None;
+    group_top: a group of neighbours scores as the sum of its so many largest choice scores; normalise: the chosen
+    experts' scores are divided by their sum; scale: a constant on the weights."""
+
+    def __init__(self, scoring: str = "softmax", correction=None, group_top: int = 1, normalise: bool = True, scale: float = 1.0):
+        if scoring not in ("softmax", "sigmoid") or group_top < 1:
+            raise ValueError("scoring is 'softmax' or 'sigmoid', group_top positive")
+        self.scoring, self.correction, self.group_top = scoring, correction, int(group_top)
+        self.normalise, self.scale = bool(normalise), float(scale)
+
+    def check(self, E: int) -> None:
+        c = self.correction
+        _check(c is None or (c.dtype == torch.float32 and c.shape == (E,) and c.is_contiguous()), "moe_route: the correction must be float32 [experts]")
+
+    def args(self) -> tuple:
+        return (self.group_top, int(self.scoring == "sigmoid"), int(self.normalise), self.scale, _ptr(self.correction))
+
+
 class HipBackend:
     """Each method is one kernel (or one dispatch among kernels of the same meaning)."""
 
     name = "hip"
 
     # -- rows ----------------------------------------------------------------------------
-    def gather_rows(self, src: torch.Tensor, idx: torch.Tensor) -> torch.Tensor:
+    def gather_rows(self, src: torch.Tensor, idx: torch.Tensor, scale: float | None = None) -> torch.Tensor:
         """out[r] = src[idx[r]] (embedding lookup: reference layers/embed_head.py:10-11;
-        rows that want logits: layers/embed_head.py:20-22)."""
+        rows that want logits: layers/embed_head.py:20-22). With `scale`: out[r] = scale * src[idx[r]] in float32
+        (embedding rows under a multiplier: they start the 32-bit stream without a rounding of their own)."""
         _check(src.dim() == 2 and src.is_contiguous(), "gather_rows: source must be a contiguous matrix")
         _check(_is_i32(idx) and idx.dim() == 1, "gather_rows: indices must be int32 [n]")
+        if scale is not None:
+            out = torch.empty((idx.numel(), src.shape[1]), dtype=torch.float32, device=src.device)
+            core().call("me_gather_rows_scaled", src.data_ptr(), _code(src.dtype), idx.data_ptr(), out.data_ptr(), idx.numel(),
+                        src.shape[1], src.shape[0], float(scale), _stream())
+            return out
         out = torch.empty((idx.numel(), src.shape[1]), dtype=src.dtype, device=src.device)
         core().call("me_gather_rows", src.data_ptr(), idx.data_ptr(), out.data_ptr(), idx.numel(),
                     src.shape[1] * src.element_size(), src.shape[0], _stream())
@@ -852,15 +881,24 @@ class HipBackend:
         return out
 
     def weighted_sum(self, terms, norm_weight=None, eps: float = 0.0, stream=None, out_dtype: torch.dtype | None = None):
-        """sum_i scale_i * (term_i + bias_i) in float32. terms: up to four (rows [T, n] in the compute dtype or float32
-        partial sums [P, T, n], a number, float32 bias [n] or None). Without `norm_weight`: returns the sum, float32
+        """sum_i scale_i * gate_i * (term_i + bias_i) in float32. terms: up to four (rows [T, n] in the compute dtype or float32
+        partial sums [P, T, n], a number, float32 bias [n] or None, and optionally gate rows: a view [T] or [T, 1] in the
+        compute dtype or float32 whose sigmoid multiplies the term token by token). Without `norm_weight`: returns the sum, float32
         [T, n]. With it (float32 [n]) and `stream` (float32 [T, n]): the norm on the sum and the residual sum in the same
         pass, stream' = stream + norm_weight * s / sqrt(mean(s^2) + eps); returns (stream' rounded to out_dtype, stream')."""
         k = len(terms)
         _check(1 <= k <= 4, "weighted_sum: one to four terms")
         T, n = terms[0][0].shape[-2:]
         ptrs, dts, parts, strides, scales, biases = (c_void_p * 4)(), (c_int * 4)(), (c_int * 4)(), (c_int64 * 4)(), (c_float * 4)(), (c_void_p * 4)()
-        for i, (t, sc, b) in enumerate(terms):
+        gates, gate_dts, gate_strides = (c_void_p * 4)(), (c_int * 4)(), (c_int64 * 4)()
+        for i, term in enumerate(terms):
+            t, sc, b = term[:3]
+            gate = term[3] if len(term) > 3 else None
+            if gate is not None:
+                _check(gate.shape[0] == T and gate.numel() == T, "weighted_sum: gate rows hold one number per token")
+                gates[i], gate_dts[i], gate_strides[i] = gate.data_ptr(), _code(gate.dtype), gate.stride(0)
+            else:
+                gates[i], gate_dts[i], gate_strides[i] = None, ME_F32, 0
             _check(t.is_contiguous() and t.shape[-2:] == (T, n) and (t.dim() == 2 or (t.dim() == 3 and t.dtype == torch.float32)),
                    "weighted_sum: a term is rows [T, n] or float32 partial sums [P, T, n]")
             _check(b is None or (b.dtype == torch.float32 and b.shape == (n,) and b.is_contiguous()), "weighted_sum: biases float32 [n]")
@@ -869,7 +907,8 @@ class HipBackend:
         dev = terms[0][0].device
         if norm_weight is None:
             out = torch.empty((T, n), dtype=torch.float32, device=dev)
-            core().call("me_weighted_sum", k, ptrs, dts, parts, strides, scales, biases, out.data_ptr(), None, 0.0, None, None, None, 0, T, n, _stream())
+            core().call("me_weighted_sum", k, ptrs, dts, parts, strides, scales, biases, out.data_ptr(), None, 0.0, None, None, None, 0, T, n,
+                        gates, gate_dts, gate_strides, _stream())
             return out
         _check(norm_weight.dtype == torch.float32 and norm_weight.shape == (n,) and norm_weight.is_contiguous()
                and stream is not None and stream.dtype == torch.float32 and stream.shape == (T, n) and stream.is_contiguous(),
@@ -878,7 +917,7 @@ class HipBackend:
         rounded = new if out_dtype in (None, torch.float32) else torch.empty((T, n), dtype=out_dtype, device=dev)
         core().call("me_weighted_sum", k, ptrs, dts, parts, strides, scales, biases, None, norm_weight.data_ptr(), float(eps),
                     stream.data_ptr(), new.data_ptr(), None if rounded is new else rounded.data_ptr(),
-                    _code(rounded.dtype), T, n, _stream())
+                    _code(rounded.dtype), T, n, gates, gate_dts, gate_strides, _stream())
         return rounded, new
 
     def token_shift(self, x, mu, state, state_slots, cu_seqlens, seq_of_token) -> torch.Tensor:
@@ -905,6 +944,7 @@ class HipBackend:
         rule "bonus":  d = exp(-exp(raw + base));  y = (S + diag(bonus) k v^T)^T q;  S <- diag(d) S + k v^T.
         rule "delta":  d = exp(-rate_h softplus(raw + base));  S <- diag(d) S;  u = sigmoid(beta) (v - S^T k);
                        S <- S + k u^T;  y = S^T q.
+        rule "gated":  d = sigmoid(raw + base) ^ rate_h;  S <- diag(d) S + k v^T;  y = S^T q.
         q, k: row views [T, G * N] (heads share them by groups of H / G); v: [T, H * P]; raw: [T, H * N]; beta: [T, H];
         base, bonus: float32 [H * N]; rate: float32 [H]. `unit_eps`: q and k are made unit vectors per head first, x /
         sqrt(sum(x^2) + unit_eps); q is multiplied by q_scale. Everything but the rows read is float32. Returns float32
@@ -918,7 +958,7 @@ class HipBackend:
                "decay_rows_recurrence: state must be float32 [slots, H * N * P]")
         for w, width in ((base, H * N), (bonus, H * N), (rate, H)):
             _check(w is None or (w.dtype == torch.float32 and w.numel() == width and w.is_contiguous()), "decay_rows_recurrence: constants float32")
-        _check(base is not None and (bonus is not None if rule == "bonus" else (rate is not None and beta is not None)),
+        _check(base is not None and (bonus is not None if rule == "bonus" else (rate is not None and (beta is not None or rule == "gated"))),
                "decay_rows_recurrence: the rule's constants are missing")
         if beta is not None:
             _check(beta.shape == (T, H) and beta.stride(1) == 1 and beta.dtype == dtype, "decay_rows_recurrence: write strengths [T, H]")
@@ -936,48 +976,56 @@ class HipBackend:
         return y
 
     # -- routed experts ------------------------------------------------------------------
-    def moe_route(self, x, router, top: int, group_count: int = 1, group_keep: int = 1):
-        """Which experts each token uses and with what weights. x: [T, n] rows; router: float32 [E, n]. Scores are the
-        softmax of router . x over all E experts, in float32. With group_count > 1 the experts form that many equal
-        groups of neighbours, a group scores as its best expert, and only experts of the group_keep best groups can be
-        chosen. The `top` largest scores are chosen (ties: the lower index); their weights are the scores divided by
-        their sum + 1e-20. Returns (ids int32 [T, top], weights float32 [T, top])."""
+    def moe_route(self, x, router, top: int, group_count: int = 1, group_keep: int = 1, rule: "RouteRule | None" = None):
+        """Which experts each token uses and with what weights. x: [T, n] rows; router: float32 [E, n]. The logits router . x
+        are float32. `rule` (a `RouteRule`; None: its defaults) says how they become scores (their softmax over all E
+        experts, or a sigmoid each), whether a correction per expert joins the scores for the choice, how a group of
+        neighbours scores (the sum of its group_top largest choice scores), and what the weights are (the chosen
+        experts' scores without the correction, divided by their sum + 1e-20 or not, times a constant). With
+        group_count > 1 only experts of the group_keep best groups can be chosen. The `top` largest choice scores are
+        chosen (ties: the lower index). Returns (ids int32 [T, top], weights float32 [T, top])."""
         T, n = x.shape
         E = router.shape[0]
+        rule = rule or RouteRule()
         _check(x.stride(1) == 1 and router.dtype == torch.float32 and router.shape == (E, n) and router.is_contiguous(),
                "moe_route: rows [T, n], router float32 [E, n]")
+        rule.check(E)
         ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
         weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
         logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
         core().call("me_moe_route", x.data_ptr(), x.stride(0), _code(x.dtype), router.data_ptr(), T, n, E, int(top), int(group_count),
-                    int(group_keep), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), 1, _stream())
+                    int(group_keep), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), 1, *rule.args(), _stream())
         return ids, weights
 
-    def route_and_run_experts(self, x, router, top: int, group_count: int, group_keep: int, gate_up, down) -> torch.Tensor:
+    def route_and_run_experts(self, x, router, top: int, group_count: int, group_keep: int, gate_up, down,
+                              rule: "RouteRule | None" = None, gated: bool = True) -> torch.Tensor:
         """`moe_route` and `routed_experts` behind it: float32 [top, T, hidden]. For the few tokens `moe_sort_chooses` admits,
         the kernel that orders the pairs by expert makes the choice itself from the router's logits: one launch less in a
         decode step's chain."""
         T, n = x.shape
         E = router.shape[0]
-        F = gate_up.shape[1] // 2
+        F = gate_up.shape[1] // 2 if gated else gate_up.shape[1]
+        rule = rule or RouteRule()
         if not (moe_sort_chooses(T, E, group_count) and x.dtype == torch.bfloat16 and n % 8 == 0 and F % 8 == 0 and x.stride(0) % 8 == 0
                 and x.data_ptr() % 16 == 0):
-            ids, weights = self.moe_route(x, router, top, group_count, group_keep)
-            return self.routed_experts(x, ids, weights, gate_up, down)
+            ids, weights = self.moe_route(x, router, top, group_count, group_keep, rule)
+            return self.routed_experts(x, ids, weights, gate_up, down, gated=gated)
         _check(x.stride(1) == 1 and router.dtype == torch.float32 and router.shape == (E, n) and router.is_contiguous(),
                "moe_route: rows [T, n], router float32 [E, n]")
+        rule.check(E)
         ids = torch.empty((T, top), dtype=torch.int32, device=x.device)
         weights = torch.empty((T, top), dtype=torch.float32, device=x.device)
         logits = torch.empty((T, E), dtype=torch.float32, device=x.device)
         core().call("me_moe_route", x.data_ptr(), x.stride(0), _code(x.dtype), router.data_ptr(), T, n, E, int(top), int(group_count),
-                    int(group_keep), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), 0, _stream())
-        return self.routed_experts(x, ids, weights, gate_up, down, choose_from=(logits, group_count, group_keep))
+                    int(group_keep), logits.data_ptr(), ids.data_ptr(), weights.data_ptr(), 0, *rule.args(), _stream())
+        return self.routed_experts(x, ids, weights, gate_up, down, choose_from=(logits, group_count, group_keep, rule), gated=gated)
 
     def routed_experts(self, x, ids, weights, gate_up, down, force_simple: bool = False, tile_rows: int | None = None,
-                       choose_from=None) -> torch.Tensor:
-        """Every token through its chosen gated experts: out[j, t] = weights[t, j] * W_down[e] (silu(W_gate[e] x_t) * (W_up[e] x_t)),
+                       choose_from=None, gated: bool = True) -> torch.Tensor:
+        """Every token through its chosen experts: out[j, t] = weights[t, j] * W_down[e] (silu(W_gate[e] x_t) * (W_up[e] x_t)),
         e = ids[t, j]: float32 [top, T, hidden], one partial sum per choice for a consumer that adds them. x: [T, K];
-        gate_up: [E, 2 F, K] (an expert's gate rows, then its up rows); down: [E, hidden, F]. bfloat16 with K and F in
+        gate_up: [E, 2 F, K] (an expert's gate rows, then its up rows); down: [E, hidden, F]. With `gated` False the experts
+        have no gate: gate_up is [E, F, K] (up rows only) and an expert is W_down[e] relu(W_up[e] x_t)^2. bfloat16 with K and F in
         whole steps of 8: the (token, choice) pairs are ordered by expert and cut into tiles that never span two experts, of
         64 rows (a workgroup's 64 x 64 tile of the matrix-core kernel) or, while an expert gets few rows (`expert_tile_rows`;
         `tile_rows` forces it), of 16 rows for the kernel that streams the chosen experts' weights with K cut over a
@@ -985,8 +1033,8 @@ class HipBackend:
         T, K = x.shape
         top = ids.shape[1]
         E, F2, _ = gate_up.shape
-        F, N = F2 // 2, down.shape[1]
-        _check(x.stride(1) == 1 and gate_up.is_contiguous() and down.is_contiguous() and gate_up.shape == (E, 2 * F, K)
+        F, N = (F2 // 2 if gated else F2), down.shape[1]
+        _check(x.stride(1) == 1 and gate_up.is_contiguous() and down.is_contiguous() and gate_up.shape == (E, (2 if gated else 1) * F, K)
                and down.shape == (E, N, F) and gate_up.dtype == x.dtype and down.dtype == x.dtype, "routed_experts: operand shapes")
         _check(ids.dtype == torch.int32 and ids.is_contiguous() and weights.dtype == torch.float32 and weights.is_contiguous()
                and ids.shape == (T, top) and weights.shape == (T, top), "routed_experts: ids int32 [T, top], weights float32 [T, top]")
@@ -998,21 +1046,61 @@ class HipBackend:
                  and not force_simple and Pn // rows + min(E, Pn) <= 65535)
         if not tiled:
             core().call("me_moe_experts_simple", x.data_ptr(), x.stride(0), _code(x.dtype), gate_up.data_ptr(), down.data_ptr(),
-                        ids.data_ptr(), weights.data_ptr(), act.data_ptr(), out.data_ptr(), T, top, N, F, K, _stream())
+                        ids.data_ptr(), weights.data_ptr(), act.data_ptr(), out.data_ptr(), T, top, N, F, K, int(gated), _stream())
             return out
         max_tiles = Pn // rows + min(E, Pn)
         meta = torch.empty((Pn + E + 1 + 2 * max_tiles,), dtype=torch.int32, device=x.device)
         order, offsets = meta[:Pn], meta[Pn:Pn + E + 1]
         tile_expert, tile_row = meta[Pn + E + 1:Pn + E + 1 + max_tiles], meta[Pn + E + 1 + max_tiles:]
-        # choose_from (logits, group_count, group_keep): ids and weights are still empty and the sort kernel fills them
-        logits, gc, gk = choose_from if choose_from is not None else (None, 1, 1)
+        # choose_from (logits, group_count, group_keep, rule): ids and weights are still empty and the sort kernel fills them
+        logits, gc, gk, rule = choose_from if choose_from is not None else (None, 1, 1, RouteRule())
         _check(choose_from is None or tiled, "routed_experts: the choice inside the sort kernel needs the tiled path")
         core().call("me_moe_sort", ids.data_ptr(), Pn, E, max_tiles, rows, order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
-                    tile_row.data_ptr(), _ptr(logits), weights.data_ptr(), top, int(gc), int(gk), _stream())
+                    tile_row.data_ptr(), _ptr(logits), weights.data_ptr(), top, int(gc), int(gk), *rule.args(), _stream())
         core().call("me_moe_gate_up", x.data_ptr(), x.stride(0), gate_up.data_ptr(), order.data_ptr(), offsets.data_ptr(),
-                    tile_expert.data_ptr(), tile_row.data_ptr(), act.data_ptr(), T, top, F, K, max_tiles, rows, _stream())
+                    tile_expert.data_ptr(), tile_row.data_ptr(), act.data_ptr(), T, top, F, K, max_tiles, rows, int(gated), _stream())
         core().call("me_moe_down", act.data_ptr(), down.data_ptr(), order.data_ptr(), offsets.data_ptr(), tile_expert.data_ptr(),
                     tile_row.data_ptr(), weights.data_ptr(), out.data_ptr(), T, top, N, F, max_tiles, rows, _stream())
+        return out
+
+    # -- attention over a latent that all heads share ------------------------------------------
+    def latent_prepare(self, rows, q_off: int, kv_off: int | None, H: int, dn: int, dr: int, R: int, D: int, norm_weight, eps: float,
+                       table, positions, slots, k_cache, v_cache, page: int) -> torch.Tensor:
+        """From the rows of a layer's packed product ([T, ...]: H query heads of dn unrotated and dr rotating dimensions from
+        column q_off; from column kv_off the latent's R rows and dr rows of a key part that all heads share): the RMS norm
+        of the latent with `norm_weight` (float32 [R]), the rotation of the shared key part and of every head's rotating
+        query part in adjacent pairs by `table` (float32 [positions, dr / 2, 2]: cos, sin), and the write into the pages at
+        `slots`: k_cache [pages, 1, page, D] takes [latent | rotated part | zeros], v_cache [pages, 1, D, page] the latent.
+        kv_off None: a layer that reads another layer's pages writes none. Returns the queries' frame [T, H * D] in the
+        rows' dtype with slots R .. R + dr of every head filled (the rotated part; zeros behind it): slots 0 .. R wait for
+        the queries carried into the latent's space (`heads_linear`)."""
+        T = rows.shape[0]
+        _check(rows.dim() == 2 and rows.stride(1) == 1 and q_off + H * (dn + dr) <= rows.shape[1], "latent_prepare: rows [T, n], unit inner stride")
+        _check(dr % 2 == 0 and D >= R + dr and (dr == 0 or (table is not None and table.dtype == torch.float32 and table.is_contiguous()
+               and table.shape[1:] == (dr // 2, 2))), "latent_prepare: the rotation's table must be float32 [positions, dr / 2, 2]")
+        _check(_is_i32(positions, T), "latent_prepare: positions must be int32")
+        write = kv_off is not None
+        if write:
+            _check(kv_off + R + dr <= rows.shape[1] and _is_i32(slots, T) and norm_weight.dtype == torch.float32 and norm_weight.shape == (R,)
+                   and norm_weight.is_contiguous(), "latent_prepare: slots int32, norm weight float32 [rank]")
+            _check(k_cache.shape[1:] == (1, page, D) and v_cache.shape[1:] == (1, D, page) and k_cache.dtype == rows.dtype
+                   and v_cache.dtype == rows.dtype, "latent_prepare: cache layout mismatch")
+        qa = torch.empty((T, H * D), dtype=rows.dtype, device=rows.device)
+        core().call("me_latent_prepare", rows.data_ptr(), rows.stride(0), _code(rows.dtype), int(q_off), int(kv_off or 0), H, dn, dr, R, D,
+                    _ptr(norm_weight) if write else None, float(eps), _ptr(table), 0 if table is None else table.shape[0],
+                    positions.data_ptr(), slots.data_ptr() if write else None, qa.data_ptr(), qa.stride(0),
+                    k_cache.data_ptr() if write else None, v_cache.data_ptr() if write else None, int(page), T, _stream())
+        return qa
+
+    def heads_linear(self, x, w, out) -> torch.Tensor:
+        """out[t, h, :] = w[h] x[t, h, :]: a product per head. x: a view [T, H, K], w: [H, N, K] contiguous, out: a view [T, H, N],
+        all of one dtype; the views' inner strides are 1, their token and head strides are free (heads inside a wider row)."""
+        T, H, K = x.shape
+        N = w.shape[1]
+        _check(w.shape == (H, N, K) and w.is_contiguous() and out.shape == (T, H, N) and x.stride(2) == 1 and out.stride(2) == 1
+               and x.dtype == w.dtype == out.dtype, "heads_linear: x [T, H, K], w [H, N, K], out [T, H, N] of one dtype")
+        core().call("me_heads_linear", x.data_ptr(), x.stride(0), x.stride(1), w.data_ptr(), out.data_ptr(), out.stride(0), out.stride(1),
+                    _code(x.dtype), T, H, N, K, _stream())
         return out
 
     # -- sampling ------------------------------------------------------------------------
@@ -1633,3 +1721,5 @@ def decay_rows_recurrence(*a, **k): return backend().decay_rows_recurrence(*a, *
 def moe_route(*a, **k): return backend().moe_route(*a, **k)
 def routed_experts(*a, **k): return backend().routed_experts(*a, **k)
 def route_and_run_experts(*a, **k): return backend().route_and_run_experts(*a, **k)
+def latent_prepare(*a, **k): return backend().latent_prepare(*a, **k)
+def heads_linear(*a, **k): return backend().heads_linear(*a, **k)

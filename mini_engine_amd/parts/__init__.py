@@ -1,4 +1,4 @@
 """Model parts. Importing this package registers the built-in parts."""
 from .base import (PAGE, CacheNeed, CacheView, FeedForward, Head, LayerCall, Mixer, Norm, PageTensor, ParamSpec, Part,  # noqa: F401
                    PendingNorm, PositionEncoding, ScaledSum, Settled, StateNeed, make_part, register_part, registered)
-from . import attention, block, embedding, feed_forward, hybrid, linear, moe, norms, recurrent, rotary  # noqa: F401
+from . import attention, block, embedding, feed_forward, hybrid, latent, linear, moe, norms, recurrent, rotary  # noqa: F401

@@ -52,6 +52,9 @@ class Attention(Mixer):
     sigmoid of further output features of the packed product, as many as the heads' values), `out_bias` (a bias on the
     output product), and `qkv_bias` together with per-head norms or a position encoding (the biases are then added to
     the packed product's unrounded sums by a kernel of their own in front of the per-head norm and rotation).
+    `qk_norm_weights=False`: the per-head norm of q and k has no learned weights (every head is brought to unit root mean
+    square and that is all). Such a norm may stand in front of the rotation or behind it: a rotation changes no pair's
+    length, so the head's mean square, and with it the result, is the same either way.
     """
 
     takes_pending_norm = True      # x goes to the packed product and nowhere else
@@ -62,7 +65,7 @@ class Attention(Mixer):
                  chunk: int | None = None, head_gate: bool = False, qkv_bias: bool = False, qk_norm_over: str = "head",
                  q_temperature: tuple | None = None, value_mix: str | None = None, value_mix_key: str = "v_first",
                  keep_first: int = 0, score_cap: float | None = None, sinks: bool = False, output_gate: bool = False,
-                 out_bias: bool = False):
+                 out_bias: bool = False, qk_norm_weights: bool = True):
         super().__init__()
         if qk_norm_over not in ("head", "projection") or value_mix not in (None, "first", "blend"):
             raise ValueError("qk_norm_over is 'head' or 'projection', value_mix None, 'first' or 'blend'")
@@ -124,7 +127,12 @@ class Attention(Mixer):
         self._relayout = self._relayout or rows % 8 != 0
         self.gate_at = self.q_size + (2 * self.kv_size if own_kv else 0)      # first gate column of the kernels' rows
         self._laid_out = False
-        if qk_norm_eps is not None:
+        self.qk_norm_weights = bool(qk_norm_weights)
+        if qk_norm_eps is not None and not self.qk_norm_weights:
+            if qk_norm_over != "head":
+                raise ValueError("a norm without weights is a norm per head")
+            self.q_norm_weight = self.k_norm_weight = None
+        elif qk_norm_eps is not None:
             whole = qk_norm_over == "projection"
             self.add_param("q_norm_weight", ParamSpec((stored_q if whole else self.stored_dim,), init="norm", dtype="float32"))
             if own_kv:
@@ -156,6 +164,9 @@ class Attention(Mixer):
 
     def finalize(self, device, dtype, max_positions):
         """The kernels' layout of the stored parameters, where it differs (see the class text)."""
+        if self.norm_eps is not None and not self.qk_norm_weights and not self._laid_out:
+            self.q_norm_weight = torch.ones(self.stored_dim, dtype=torch.float32, device=device)
+            self.k_norm_weight = torch.ones(self.stored_dim, dtype=torch.float32, device=device) if self.own_kv else None
         if not self._relayout or self._laid_out:
             return
         H, G, D, n, nv = self.num_heads, self.num_kv_heads, self.head_dim, self.stored_dim, self.value_dim

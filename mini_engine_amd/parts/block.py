@@ -42,12 +42,18 @@ class PreNormBlock(Part):
     norm call). The residual stream is float32.
     """
 
-    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm, feed_forward: FeedForward):
+    def __init__(self, norm1: Norm, mixer: Mixer, norm2: Norm | None, feed_forward: FeedForward | None):
+        """Without a feed-forward (and its norm) the layer is its first half: the mixer's output is what is left to add."""
         super().__init__()
+        if (norm2 is None) != (feed_forward is None):
+            raise ValueError("a feed-forward and its norm come together")
         self.add_child("norm1", norm1)
         self.add_child("mixer", mixer)
-        self.add_child("norm2", norm2)
-        self.add_child("feed_forward", feed_forward)
+        if feed_forward is not None:
+            self.add_child("norm2", norm2)
+            self.add_child("feed_forward", feed_forward)
+        else:
+            self.norm2 = self.feed_forward = None
 
     def cache_need(self):
         return self.mixer.cache_need()
@@ -67,6 +73,8 @@ class PreNormBlock(Part):
         else:
             x, residual = norm_of(self.norm1, h, residual)
             a = self.mixer.forward(x, step, cache, state)
+        if self.feed_forward is None:
+            return a, residual
         if getattr(self.feed_forward, "takes_pending_norm", False):
             x = PendingNorm(self.norm2, a, residual)
             out = self.feed_forward.forward(x)

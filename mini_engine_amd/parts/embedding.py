@@ -8,14 +8,16 @@ from .base import Head, ParamSpec, Part
 
 
 class TokenEmbedding(Part):
-    def __init__(self, vocab_size: int, hidden_size: int):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float | None = None):
+        """`scale`: the rows are multiplied by it and come back in float32 (they start the 32-bit stream unrounded)."""
         super().__init__()
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
+        self.scale = None if scale is None else float(scale)
         self.add_param("weight", ParamSpec((vocab_size, hidden_size), init="matrix", dtype="compute"))
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
-        return ops.gather_rows(self.weight, token_ids)
+        return ops.gather_rows(self.weight, token_ids) if self.scale is None else ops.gather_rows(self.weight, token_ids, scale=self.scale)
 
 
 class LMHead(Head):

@@ -93,6 +93,11 @@ def _half(shape, generator, device):
     return torch.rand(shape, generator=generator, dtype=torch.float32, device=device)
 
 
+def _decay_bias(shape, generator, device):
+    """Biases of a sigmoid decay spread over 1..5: per-step decays between 0.73 and 0.993 before the temperature."""
+    return 1.0 + 4.0 * torch.rand(shape, generator=generator, dtype=torch.float32, device=device)
+
+
 def _bonus(shape, generator, device):
     return torch.rand(shape, generator=generator, dtype=torch.float32, device=device) - 0.5
 
@@ -224,3 +229,54 @@ def _rows(rows: torch.Tensor, start: int, width: int) -> torch.Tensor:
     if (start * rows.element_size()) % 16 == 0 and (rows.stride(0) * rows.element_size()) % 16 == 0:
         return view
     return view.contiguous()
+
+
+@register_part("mixer", "gla")
+class GatedLinearAttention(Mixer):
+    """Linear attention whose state rows decay each at a rate the token chooses, without a bonus and without a shift:
+    q = W_q x * key_dim^(-1/2), k = W_k x ([heads, key_dim]), v = W_v x ([heads, value_dim]); the decay of every key
+    channel alpha = sigmoid(W_a2 (W_a1 x) + bias) ^ (1 / tau) (a thin matrix pair). Per head
+        S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,      o_t = S_t^T q_t.
+    Every head's o is divided by its root mean square and multiplied by a weight of the value size that the heads share;
+    the heads side by side are multiplied by silu(W_g x) and projected. q, k, v, the gate and the pair's first matrix are
+    one packed product. The decay and everything behind it is float32; a request's state row holds the heads' matrices."""
+
+    takes_pending_norm = True      # x goes to the packed product and nowhere else
+
+    def __init__(self, hidden_size: int, num_heads: int, key_dim: int, value_dim: int, decay_rank: int, tau: float, norm_eps: float):
+        super().__init__()
+        if not tau > 0:
+            raise ValueError("the decay's temperature must be positive")
+        self.hidden_size, self.num_heads, self.key_dim, self.value_dim = hidden_size, num_heads, key_dim, value_dim
+        self.decay_rank, self.tau, self.norm_eps = decay_rank, float(tau), float(norm_eps)
+        qk, inner = num_heads * key_dim, num_heads * value_dim
+        self.qk, self.inner = qk, inner
+        self.add_child("in_proj", Linear(hidden_size, 2 * qk + 2 * inner + decay_rank,
+                                         parts={"q": qk, "k": qk, "v": inner, "g": inner, "a1": decay_rank}))
+        self.add_child("a2", Linear(decay_rank, qk))
+        self.add_param("a2_bias", ParamSpec((qk,), init=_decay_bias, dtype="float32"))
+        self.add_param("norm_weight", ParamSpec((value_dim,), init="norm", dtype="float32"))
+        self.add_child("o", Linear(inner, hidden_size))
+        self._rate = self._norm = None
+
+    def state_need(self):
+        return StateNeed((self.num_heads * self.key_dim * self.value_dim,), "float32")
+
+    def set_param(self, local, tensor):
+        super().set_param(local, tensor)
+        self._rate = None
+
+    def finalize(self, device, dtype, max_positions):
+        self._rate = torch.full((self.num_heads,), 1.0 / self.tau, dtype=torch.float32, device=device)
+        self._norm = self.norm_weight.repeat(self.num_heads).contiguous()         # one weight for every head's values
+
+    def forward(self, x, step, cache, state):
+        H, N, P, qk, inner = self.num_heads, self.key_dim, self.value_dim, self.qk, self.inner
+        rows = self.in_proj.forward(x)                                            # [T, q | k | v | g | a1]
+        raw = self.a2.forward(rows[:, 2 * qk + 2 * inner:])
+        y = ops.decay_rows_recurrence(rows[:, :qk], rows[:, qk:2 * qk], rows[:, 2 * qk:2 * qk + inner], raw, state, step.state_slots,
+                                      step.cu_seqlens, step.q_lens, H, H, N, P, "gated", base=self.a2_bias, rate=self._rate,
+                                      q_scale=N ** -0.5)
+        g = rows[:, 2 * qk + inner:2 * qk + 2 * inner]
+        o = ops.gated_rms_norm(y, g, self._norm, self.norm_eps, H, "silu_behind", g.dtype)
+        return self.o.forward(o, allow_partials=True)

@@ -55,4 +55,4 @@ def build_model(model_config, checkpoint_names=None, checkpoint_shapes=None):
 
 
 def _load_builtin() -> None:
-    from .models import negosun, qwen3, sigosun, tavevik  # noqa: F401  (they register themselves)
+    from .models import goluzen, negosun, qwen3, sigosun, tavevik  # noqa: F401  (they register themselves)

@@ -13,7 +13,9 @@ from __future__ import annotations
 import torch
 
 
-def gather_rows(src, idx):
+def gather_rows(src, idx, scale=None):
+    if scale is not None:
+        return src[idx.long()].float() * scale
     return src[idx.long()].clone()
 
 
@@ -182,7 +184,10 @@ def add_rms_norm(y, weight, eps, stream, out_dtype):
 
 def activation(x, kind):
     v = x.float()
-    v = v * torch.sigmoid(v) if kind == "silu" else (torch.tanh(v) if kind == "tanh" else torch.relu(v) ** 2)
+    if kind == "gelu_tanh":
+        v = 0.5 * v * (1.0 + torch.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3)))
+    else:
+        v = v * torch.sigmoid(v) if kind == "silu" else (torch.tanh(v) if kind == "tanh" else torch.relu(v) ** 2)
     return v.to(x.dtype)
 
 
@@ -283,10 +288,13 @@ def glu_clamped(gu, limit, alpha):
 
 def weighted_sum(terms, norm_weight=None, eps=0.0, stream=None, out_dtype=None):
     total = None
-    for t, sc, b in terms:
+    for term in terms:
+        t, sc, b = term[:3]
         v = t.float().sum(0) if t.dim() == 3 else t.float()
         if b is not None:
             v = v + b
+        if len(term) > 3 and term[3] is not None:
+            v = v * torch.sigmoid(term[3].float().reshape(-1, 1))
         total = sc * v if total is None else total + sc * v
     if norm_weight is None:
         return total
@@ -334,6 +342,10 @@ def decay_rows_recurrence(q, k, v, raw, state, state_slots, cu_seqlens, q_lens, 
                 kv = kt[:, :, None] * vt[:, None, :]
                 out = torch.einsum("hnp,hn->hp", S + bonus.view(H, N)[:, :, None] * kv, qt)
                 S = d[:, :, None] * S + kv
+            elif rule == "gated":
+                d = torch.exp(-rate[:, None] * softplus(-z))          # sigmoid(z) ^ rate
+                S = d[:, :, None] * S + kt[:, :, None] * vt[:, None, :]
+                out = torch.einsum("hnp,hn->hp", S, qt)
             else:
                 d = torch.exp(-rate[:, None] * softplus(z))
                 S = d[:, :, None] * S
@@ -391,45 +403,84 @@ def qkv_prepare_store(rows, bias, q_weight, k_weight, eps, nq, nk, temperature, 
     return q.to(dt).contiguous()
 
 
-def moe_route(x, router, top, group_count=1, group_keep=1):
+def moe_route(x, router, top, group_count=1, group_keep=1, rule=None):
     z = x.float() @ router.float().t()
-    s = torch.softmax(z, dim=-1)
+    sigmoid = rule is not None and rule.scoring == "sigmoid"
+    s = torch.sigmoid(z) if sigmoid else torch.softmax(z, dim=-1)
     T, E = s.shape
-    m = s.clone()
+    m = s.clone() if rule is None or rule.correction is None else s + rule.correction
     if group_count > 1 and group_keep < group_count:
         per = E // group_count
-        gs = s.view(T, group_count, per).amax(-1)
+        count = min(1 if rule is None else rule.group_top, per)
+        gs = m.view(T, group_count, per).topk(count, -1).values.sum(-1)
         kept = torch.zeros((T, group_count), dtype=torch.bool, device=x.device)
         for _ in range(group_keep):
-            best = torch.where(kept, torch.full_like(gs, -2.0), gs).argmax(-1)      # ties: the lower index
+            best = torch.where(kept, torch.full_like(gs, -float("inf")), gs).argmax(-1)      # ties: the lower index
             kept[torch.arange(T), best] = True
-        m = torch.where(kept.repeat_interleave(per, 1), m, torch.full_like(m, -1.0))
+        m = torch.where(kept.repeat_interleave(per, 1), m, torch.full_like(m, -float("inf")))
     ids = torch.empty((T, top), dtype=torch.int64, device=x.device)
     for j in range(top):
         best = m.argmax(-1)
         ids[:, j] = best
-        m[torch.arange(T), best] = -2.0
+        m[torch.arange(T), best] = -float("inf")
     w = torch.gather(s, 1, ids)
-    return ids.to(torch.int32), (w / (w.sum(-1, keepdim=True) + 1e-20)).float()
+    if rule is None or rule.normalise:
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    return ids.to(torch.int32), (w * (1.0 if rule is None else rule.scale)).float()
 
 
-def route_and_run_experts(x, router, top, group_count, group_keep, gate_up, down):
-    ids, weights = moe_route(x, router, top, group_count, group_keep)
-    return routed_experts(x, ids, weights, gate_up, down)
+def route_and_run_experts(x, router, top, group_count, group_keep, gate_up, down, rule=None, gated=True):
+    ids, weights = moe_route(x, router, top, group_count, group_keep, rule)
+    return routed_experts(x, ids, weights, gate_up, down, gated=gated)
 
 
-def routed_experts(x, ids, weights, gate_up, down, force_simple=False, tile_rows=None, choose_from=None):
+def routed_experts(x, ids, weights, gate_up, down, force_simple=False, tile_rows=None, choose_from=None, gated=True):
     T, K = x.shape
     top = ids.shape[1]
-    F = gate_up.shape[1] // 2
+    F = gate_up.shape[1] // 2 if gated else gate_up.shape[1]
     out = torch.zeros((top, T, down.shape[1]), dtype=torch.float32, device=x.device)
     xf = x.float()
     for j in range(top):
         for e in ids[:, j].unique().tolist():
             rows = (ids[:, j] == e).nonzero().flatten()
             gu = xf[rows] @ gate_up[e].float().t()
-            act = (gu[:, :F] * torch.sigmoid(gu[:, :F]) * gu[:, F:]).to(x.dtype).float()
-            out[j, rows] = (act @ down[e].float().t()) * weights[rows, j][:, None]
+            act = gu[:, :F] * torch.sigmoid(gu[:, :F]) * gu[:, F:] if gated else torch.relu(gu) ** 2
+            out[j, rows] = (act.to(x.dtype).float() @ down[e].float().t()) * weights[rows, j][:, None]
+    return out
+
+
+def latent_prepare(rows, q_off, kv_off, H, dn, dr, R, D, norm_weight, eps, table, positions, slots, k_cache, v_cache, page):
+    T = rows.shape[0]
+    qa = torch.zeros((T, H, D), dtype=rows.dtype, device=rows.device)
+    cs = table[positions.long()] if dr else None                      # [T, dr / 2, 2]
+
+    def turn(x):                                                      # [..., dr] in adjacent pairs
+        u, v = x[..., 0::2].float(), x[..., 1::2].float()
+        c, s = cs[..., 0], cs[..., 1]
+        while c.dim() < u.dim():
+            c, s = c.unsqueeze(1), s.unsqueeze(1)
+        out = torch.empty_like(x, dtype=torch.float32)
+        out[..., 0::2], out[..., 1::2] = u * c - v * s, v * c + u * s
+        return out
+
+    q = rows[:, q_off:q_off + H * (dn + dr)].reshape(T, H, dn + dr)
+    if dr:
+        qa[:, :, R:R + dr] = turn(q[:, :, dn:]).to(rows.dtype)
+    if kv_off is not None:
+        kv = rows[:, kv_off:kv_off + R + dr].float()
+        c = kv[:, :R] * torch.rsqrt(kv[:, :R].pow(2).mean(-1, keepdim=True) + eps) * norm_weight
+        key = torch.zeros((T, 1, D), dtype=torch.float32, device=rows.device)
+        key[:, 0, :R] = c
+        if dr:
+            key[:, 0, R:R + dr] = turn(kv[:, R:])
+        val = torch.zeros((T, 1, D), dtype=torch.float32, device=rows.device)
+        val[:, 0, :R] = c
+        write_pages(key.to(rows.dtype), val.to(rows.dtype), slots, k_cache, v_cache, page)
+    return qa.view(T, H * D)
+
+
+def heads_linear(x, w, out):
+    out.copy_(torch.einsum("thk,hnk->thn", x.float(), w.float()).to(out.dtype))
     return out
 
 
@@ -518,3 +569,5 @@ class PlainBackend:
     moe_route = staticmethod(moe_route)
     routed_experts = staticmethod(routed_experts)
     route_and_run_experts = staticmethod(route_and_run_experts)
+    latent_prepare = staticmethod(latent_prepare)
+    heads_linear = staticmethod(heads_linear)
