@@ -418,18 +418,19 @@ def other_size(run: dict, context: int) -> dict:
 
 
 def design_comparison(args) -> int:
-    """`--design`: the design and Qwen3 side by side at each named size, one JSON line."""
+    """`--design`: the design and Qwen3 (or the design named by `--beside`) side by side at each named size, one JSON line."""
     points = [int(p) for p in args.points.split(",") if p and int(p) != args.batch]
     steps, warmup = min(args.steps, 32), min(args.warmup, 4)
     rows = {}
     with tempfile.TemporaryDirectory() as tmp:
         for size in [s for s in args.design_sizes.split(",") if s]:
             pair = {}
-            for name, which in ((args.design, f"{args.design}:{size}"), ("qwen3", size)):
+            other = size if args.beside == "qwen3" else f"{args.beside}:{size}"
+            for name, which in ((args.design, f"{args.design}:{size}"), (args.beside, other)):
                 run = measure(args, which, args.layers, tmp, [args.batch] + points, steps, warmup)
                 pair[name] = other_size(run, args.context)
             rows[size] = pair
-    line = {"metric": f"{args.design} beside qwen3: prefill tok/s at {args.prefill_tokens} tokens, decode tok/s at batch "
+    line = {"metric": f"{args.design} beside {args.beside}: prefill tok/s at {args.prefill_tokens} tokens, decode tok/s at batch "
                       f"{args.batch}/{'/'.join(map(str, points))}", "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
             "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: seeded random token ids and weights",
             "sizes": rows}
@@ -471,7 +472,9 @@ def main(argv=None) -> int:
     ap.add_argument("--no-graphs", action="store_true", help="launch decode kernels one by one instead of replaying HIP graphs")
     ap.add_argument("--no-run-ahead", action="store_true",
                     help="fetch every decode step's tokens before the next step is launched")
-    ap.add_argument("--design", default=None, choices=["sigosun", "negosun", "tavevik"],
+    ap.add_argument("--beside", default="qwen3", choices=["qwen3", "sigosun", "negosun", "tavevik", "goluzen"],
+                    help="with --design: the model the design is measured beside, at the same width, depth and vocabulary")
+    ap.add_argument("--design", default=None, choices=["sigosun", "negosun", "tavevik", "goluzen"],
                     help="instead of the default workload: prefill and decode throughput of this design at the layer sizes "
                          "named by --design-sizes (random weights), each beside Qwen3 at the same width, depth and vocabulary")
     ap.add_argument("--design-sizes", default="0.6b,8b")

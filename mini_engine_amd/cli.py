@@ -71,7 +71,7 @@ def main(argv=None) -> int:
         try:
             cfg, _ = named_config(args.random_weights)
         except KeyError:
-            p.error(f"--random-weights must be one of {sorted(SIZES)}, or sigosun:<size> / negosun:<size> / tavevik:<size> for those designs at those layer sizes")
+            p.error(f"--random-weights must be one of {sorted(SIZES)}, or sigosun:<size> / negosun:<size> / tavevik:<size> / goluzen:<size> for those designs at those layer sizes")
         tmp = tempfile.TemporaryDirectory()
         path = write_random_model(cfg, args.seed, tmp.name)
     path = os.path.expanduser(path)

@@ -3,7 +3,7 @@ with random weights (no model folder at hand). The figures are those of the publ
 files; a model folder's own config.json always wins where there is one."""
 from __future__ import annotations
 
-from .model_config import NegosunConfig, Qwen3Config, SigosunConfig, TavevikConfig
+from .model_config import GoluzenConfig, NegosunConfig, Qwen3Config, SigosunConfig, TavevikConfig
 
 SIZES = {
     # name: (layers, hidden, q heads, kv heads, head_dim, intermediate, vocab, tied)
@@ -101,12 +101,55 @@ def tavevik_config(size: str, layers: int | None = None):
                                     "layers": [two if i % 2 == 0 else one for i in range(n)], "max_position_embeddings": 40960}), L
 
 
+def goluzen_config(size: str, layers: int | None = None):
+    """(a Goluzen configuration whose layers resemble that size's: the same width, vocabulary and attention heads, with
+    `layers` layers or as many as the size has; that count). The mixers take turns: attention (a window of 1,024 positions
+    with 16 kept ones, half of each head turning under positions stretched fourfold, a cap of 50, sinks), attention over a
+    latent of one and a half head sizes with a rotating part of half a head size under a window of 2,048 positions,
+    linear attention with a quarter of the heads and values twice as wide as keys, attention again, latent attention on
+    the latent of the layer three before it, linear attention. The first layer's feed-forward is dense; the others have 32
+    experts of an eighth of the size's feed-forward width in four groups of which two are kept, four experts per token,
+    and a shared expert of half that width."""
+    L, h, Hq, Hkv, D, I, V, _ = SIZES[size]
+    n = layers or L
+    small = D < 64
+    attention = {"type": "attention",
+                 "mixer": {"heads": Hq, "kv_heads": Hkv, "dim": D, "vdim": D, "scale": D ** -0.5, "softcap": 50.0,
+                           "rot": {"dims": D // 2, "base": 1e6, "scaling": {"factor": 4.0}}, "mask": {"size": 1024, "keep_first": 16}}}
+    latent = lambda src: {"type": "latent_attention",
+                          "mixer": dict({"heads": Hq, "dim": D, "rot_dim": D // 2, "vdim": D, "kv_rank": 3 * D // 2, "scale": (3 * D // 2) ** -0.5,
+                                         "rot": {"dims": D // 2, "base": 1e6, "scaling": {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}},
+                                         "mask": {"size": 2048}}, **({} if src is None else {"kv_from": src}))}
+    linear = {"type": "gla", "mixer": {"heads": max(1, Hq // 4), "dim": D, "vdim": 2 * D, "tau": 16.0, "decay_rank": 8 if small else 16}}
+    moe = {"kind": "moe", "expert": {"ff": max(8, I // 8)}, "shared": {"ff": max(8, I // 2)},
+           "router": {"experts": 32, "top": 4, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
+    out, last_own = [], None
+    for i in range(n):
+        turn = i % 6
+        if turn in (0, 3):
+            entry = attention
+        elif turn in (2, 5):
+            entry = linear
+        elif turn == 1 or last_own is None:
+            entry, last_own = latent(None), i
+        else:
+            entry = latent(last_own)
+        out.append(dict(entry, mlp={"kind": "dense", "ff": I} if i == 0 else moe))
+    return GoluzenConfig.from_dict({"architecture": "Goluzen", "vocab": V, "width": h, "norm": {"eps": 1e-6}, "embedding": {"scale": 8.0},
+                                    "layers": out, "max_position_embeddings": 40960}), L
+
+
+DESIGNS = ("sigosun", "negosun", "tavevik", "goluzen")
+
+
 def named_config(name: str, layers: int | None = None):
     """(configuration, full layer count) of a name the command lines take for random weights: a Qwen3 size
-    ("0.6b"), or "sigosun:<size>" / "negosun:<size>" / "tavevik:<size>" for those designs at that size's layer sizes."""
+    ("0.6b"), or "<design>:<size>" for one of `DESIGNS` at that size's layer sizes."""
     design, _, size = name.rpartition(":")
-    if size not in SIZES or design not in ("", "qwen3", "sigosun", "negosun", "tavevik"):
-        raise KeyError(f"{name!r} is not one of {sorted(SIZES)}, optionally behind 'sigosun:', 'negosun:' or 'tavevik:'")
+    if size not in SIZES or design not in ("", "qwen3") + DESIGNS:
+        raise KeyError(f"{name!r} is not one of {sorted(SIZES)}, optionally behind one of {[d + ':' for d in DESIGNS]}")
+    if design == "goluzen":
+        return goluzen_config(size, layers)
     if design == "negosun":
         return negosun_config(size, layers)
     if design == "tavevik":

@@ -70,17 +70,21 @@ def attention(h, w, pre, m, eps):
     q = (h @ w[pre + "q"].T + w[pre + "q.b"]).view(T, H, D)
     k = (h @ w[pre + "k"].T + w[pre + "k.b"]).view(T, G, D)
     v = (h @ w[pre + "v"].T + w[pre + "v.b"]).view(T, G, Dv)
-    rot = m["rot"]
-    f = linear_frequencies(rot["dims"], rot["base"], rot["scaling"]["factor"])
-    q = unit_rms(rotate(q, pos, f, rot["dims"], False), eps)
-    k = unit_rms(rotate(k, pos, f, rot["dims"], False), eps)
+    rot = m.get("rot")
+    if rot:
+        f = linear_frequencies(rot["dims"], rot["base"], (rot.get("scaling") or {}).get("factor", 1.0))
+        q, k = rotate(q, pos, f, rot["dims"], False), rotate(k, pos, f, rot["dims"], False)
+    q, k = unit_rms(q, eps), unit_rms(k, eps)
     i, j = pos[:, None], pos[None, :]
-    seen = (j <= i) & ((i - j < m["mask"]["size"]) | (j < m["mask"]["keep_first"]))
+    seen = j <= i
+    if m.get("mask"):
+        seen = seen & ((i - j < m["mask"]["size"]) | (j < m["mask"].get("keep_first", 0)))
     out = torch.zeros(T, H, Dv, dtype=F64)
     for head in range(H):
         kv = head // (H // G)
         s = (q[:, head] @ k[:, kv].T) * m["scale"]
-        s = m["softcap"] * torch.tanh(s / m["softcap"])
+        if m.get("softcap"):
+            s = m["softcap"] * torch.tanh(s / m["softcap"])
         s = s.masked_fill(~seen, -math.inf)
         sink = w[pre + "sink"][head]
         top = torch.maximum(s.max(-1, keepdim=True).values, sink)
@@ -89,13 +93,20 @@ def attention(h, w, pre, m, eps):
     return out.reshape(T, H * Dv) @ w[pre + "o"].T
 
 
+def latent_frequencies(m):
+    sc = m["rot"].get("scaling")
+    if sc:
+        return yarn_frequencies(m["rot_dim"], m["rot"]["base"], sc)
+    return linear_frequencies(m["rot_dim"], m["rot"]["base"], 1.0), 1.0
+
+
 def latent_of(h, w, pre, m, eps):
     """What a latent-attention layer caches: the normed latent and the rotated key part that all heads share."""
     T = h.shape[0]
     R, r = m["kv_rank"], m["rot_dim"]
     rows = h @ w[pre + "dkv"].T
     c = unit_rms(rows[:, :R], eps) * w[pre + "dkv.norm"]
-    f, mult = yarn_frequencies(r, m["rot"]["base"], m["rot"]["scaling"])
+    f, mult = latent_frequencies(m)
     shared = rotate(rows[:, R:].view(T, 1, r), torch.arange(T), f, r, True, mult)[:, 0]
     return c, shared
 
@@ -106,13 +117,13 @@ def latent_attention(h, w, pre, m, eps, cached):
     H, D, r, Dv, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
     c, shared = cached
     q = (h @ w[pre + "q"].T).view(T, H, D + r)
-    f, mult = yarn_frequencies(r, m["rot"]["base"], m["rot"]["scaling"])
+    f, mult = latent_frequencies(m)
     q_rot = rotate(q[..., D:], torch.arange(T), f, r, True, mult)
     keys = (c @ w[pre + "uk"].T).view(T, H, D)
     values = (c @ w[pre + "uv"].T).view(T, H, Dv)
     pos = torch.arange(T)
     d = pos[:, None] - pos[None, :]
-    seen = (d >= 0) & (d < m["mask"]["size"])
+    seen = (d >= 0) & (d < m["mask"]["size"]) if m.get("mask") else d >= 0
     out = torch.zeros(T, H, Dv, dtype=F64)
     for head in range(H):
         s = (q[:, head, :D] @ keys[:, head].T + q_rot[:, head] @ shared.T) * m["scale"]
@@ -154,14 +165,14 @@ def choose_experts(z, correction, r):
     E, top = r["experts"], r["top"]
     s = torch.sigmoid(z)
     choice = s + correction
-    groups, keep = r["groups"]["count"], r["groups"]["keep"]
+    groups, keep = (r["groups"]["count"], r["groups"]["keep"]) if r.get("groups") else (1, 1)
     per = E // groups
     score = choice.view(-1, groups, per).topk(min(2, per), -1).values.sum(-1)
     kept = torch.zeros_like(score, dtype=torch.bool)
     kept.scatter_(1, score.topk(keep, -1).indices, True)
     eligible = kept[:, :, None].expand(-1, -1, per).reshape(-1, E)
     ids = choice.masked_fill(~eligible, -math.inf).topk(top, -1).indices
-    return ids, s.gather(1, ids) * r["scale"]
+    return ids, s.gather(1, ids) * r.get("scale", 1.0)
 
 
 def mixture(h, w, pre, f):
@@ -183,7 +194,7 @@ def forward(config, weights, tokens, keep_layers: bool = False):
     """tokens: a list of ids -> logits [T, vocab] (and the stream after every layer, [layers, T, width])."""
     w = {k: (v.to(F64) if v.is_floating_point() else v) for k, v in weights.items()}
     eps = config["norm"]["eps"]
-    x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * config["embedding"]["scale"]
+    x = w["embed"][torch.as_tensor(tokens, dtype=torch.long)] * (config.get("embedding") or {}).get("scale", 1.0)
     latents, after = {}, []
     for i, layer in enumerate(config["layers"]):
         m, pre = layer["mixer"], f"l{i}.mix."
@@ -207,3 +218,19 @@ def forward(config, weights, tokens, keep_layers: bool = False):
         after.append(x)
     logits = layer_norm(x, w["final.norm"], eps) @ w["head"].T
     return (logits, torch.stack(after)) if keep_layers else logits
+
+
+def read_folder(folder: str):
+    """(config.json as a dictionary, the checkpoint's tensors by name) of a model folder."""
+    import json
+    import os
+
+    from safetensors.torch import load_file
+
+    with open(os.path.join(folder, "config.json")) as f:
+        config = json.load(f)
+    return config, load_file(os.path.join(folder, "model.safetensors"))
+
+
+def logits(config, weights, tokens):
+    return forward(config, weights, tokens)
