@@ -33,7 +33,7 @@ CORE_SOURCES = ["elementwise.hip", "rope_kv.hip", "attention_simple.hip",
 ATTN_SOURCE = "attention_mfma.hip"
 HEADERS = ["common.h", "errors.inc", "sampling.h"]
 # Head sizes that build_all() compiles ahead of use; any other multiple of 16 up to 512 is compiled when a model first needs it.
-DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128)
+DEFAULT_HEAD_DIMS = (16, 32, 48, 64, 80, 128, 256)
 CAPPED_HEAD_DIMS = (32, 64, 128)          # ... of the variant with a cap on the scores
 
 _locks: dict = {}
