@@ -5,9 +5,10 @@
 //                    the write into the pages: the key page takes [latent | rotated part | zeros], the value page
 //                    (transposed inside a page) the latent. One pass, norm and angles in float32.
 //   heads_linear     y[t, h, :] = W[h] x[t, h, :]: a product per head (queries into the latent's space, attention
-//                    results out of it). bfloat16: 16 x 16 tiles of v_mfma_f32_16x16x32_bf16, a wave per tile, operands
-//                    straight from memory; float32, and sizes whose rows are no whole 16-byte pieces: one thread per
-//                    output, a sequential sum over K.
+//                    results out of it). bfloat16, v_mfma_f32_16x16x32_bf16: for few tokens a wave per 16 x 16 tile with
+//                    operands straight from memory; from 256 tokens on a workgroup keeps its head's matrix in LDS and
+//                    every token row is read once; float32, and sizes whose rows are no whole 16-byte pieces: one
+//                    thread per output, a sequential sum over K.
 //
 // Attention itself is the paged kernels' business: with the queries carried into the latent's space, every head
 // reads the same keys ([latent | rotated part]) and values (the latent), a single key/value head of size
@@ -138,6 +139,71 @@ __global__ void __launch_bounds__(256) heads_linear_mfma_kernel(HeadsArgs a) {
     if (n0 + 4 * g + q < a.N) o[n0 + 4 * g + q] = from_f32<bf16_t>(acc[q]);
 }
 
+// Many tokens: a workgroup stages its head's whole matrix in LDS once (rows 16 bytes apart from a multiple of 128 bytes, so
+// that the 16 lanes of an operand read touch all banks) and its 4 waves walk tiles of 16 tokens: a wave holds its tile's
+// rows in registers (K32 steps of 32) and runs down the matrix's rows 16 at a time. Tokens are read once and results written
+// once, 8 bytes a lane where the output's strides allow.
+template <int K32>
+__global__ void __launch_bounds__(256) heads_linear_lds_kernel(HeadsArgs a, int tiles_per_wave, int wide_stores) {
+  extern __shared__ __align__(16) unsigned char hl_lds[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int n = lane & 15, g = lane >> 4;
+  const int h = blockIdx.y;
+  const int KP = (a.K + 31) / 32 * 32, ld = KP + 8, NP = (a.N + 15) / 16 * 16, pieces = KP / 8;
+  const bf16_t* w = (const bf16_t*)a.w + (int64_t)h * a.N * a.K;
+  for (int i = threadIdx.x; i < NP * pieces; i += 256) {
+    const int r = i / pieces, c = i - r * pieces;
+    const uint4 v = (r < a.N && 8 * c < a.K) ? *reinterpret_cast<const uint4*>(w + (int64_t)r * a.K + 8 * c) : make_uint4(0u, 0u, 0u, 0u);
+    *reinterpret_cast<uint4*>(hl_lds + ((size_t)r * ld + 8 * c) * 2) = v;
+  }
+  __syncthreads();
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const int64_t first = ((int64_t)blockIdx.x * 4 + wave) * 16 * tiles_per_wave;
+  for (int tile = 0; tile < tiles_per_wave; ++tile) {
+    const int64_t t0 = first + 16 * tile;
+    if (t0 >= a.T) break;
+    const int64_t t = min(t0 + n, a.T - 1);
+    const bf16_t* xr = (const bf16_t*)a.x + t * a.x_stride + (int64_t)h * a.x_head + 8 * g;
+    bf16x8 xb[K32];
+#pragma unroll
+    for (int i = 0; i < K32; ++i) xb[i] = 32 * i + 8 * g < a.K ? *reinterpret_cast<const bf16x8*>(xr + 32 * i) : zero;
+    bf16_t* o = (bf16_t*)a.y + (t0 + n) * a.y_stride + (int64_t)h * a.y_head;
+    for (int n0 = 0; n0 < a.N; n0 += 16) {
+      const unsigned char* wr = hl_lds + ((size_t)(n0 + n) * ld + 8 * g) * 2;
+      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < K32; ++i)
+        if (32 * i < KP) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(*reinterpret_cast<const bf16x8*>(wr + 64 * i), xb[i], acc, 0, 0, 0);
+      if (t0 + n >= a.T) continue;
+      const int f = n0 + 4 * g;
+      if (wide_stores && f + 3 < a.N) {
+        bf16x4 r;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) r[q] = from_f32<bf16_t>(acc[q]);
+        *reinterpret_cast<bf16x4*>(o + f) = r;
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (f + q < a.N) o[f + q] = from_f32<bf16_t>(acc[q]);
+      }
+    }
+  }
+}
+
+template <int K32>
+static int launch_heads_lds(const HeadsArgs& a, size_t lds, int tiles, int wide, hipStream_t stream) {
+  static bool allowed = false;
+  if (!allowed && lds > 48 * 1024) {
+    hipError_t err = hipFuncSetAttribute((const void*)heads_linear_lds_kernel<K32>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+    ME_CHECK(err == hipSuccess, "heads_linear: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(err));
+    allowed = true;
+  }
+  const int64_t per_group = 64ll * tiles;
+  heads_linear_lds_kernel<K32><<<dim3((unsigned)((a.T + per_group - 1) / per_group), (unsigned)a.H), dim3(256), lds, stream>>>(a, tiles, wide);
+  ME_LAUNCH_CHECK();
+  return 0;
+}
+
 template <typename TX>
 __global__ void __launch_bounds__(256) heads_linear_simple_kernel(HeadsArgs a) {
   const int64_t total = a.T * a.H * a.N;
@@ -163,6 +229,15 @@ extern "C" int me_heads_linear(const void* x, int64_t x_stride, int64_t x_head, 
   a.T = T; a.H = H; a.N = N; a.K = K;
   const bool pieces = K % 8 == 0 && x_stride % 8 == 0 && x_head % 8 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
                       reinterpret_cast<uintptr_t>(w) % 16 == 0;
+  const size_t lds = (size_t)((N + 15) / 16 * 16) * ((K + 31) / 32 * 32 + 8) * 2;
+  if (dtype == ME_BF16 && pieces && T >= 256 && K <= 512 && lds <= 128 * 1024) {
+    // as many tokens to a workgroup as still leave about a thousand workgroups
+    const int tiles = T * H <= 65536 ? 1 : (T * H <= 131072 ? 2 : 4);
+    const int wide = y_stride % 4 == 0 && y_head % 4 == 0 && reinterpret_cast<uintptr_t>(y) % 8 == 0;
+    if (K <= 128) return launch_heads_lds<4>(a, lds, tiles, wide, stream);
+    if (K <= 256) return launch_heads_lds<8>(a, lds, tiles, wide, stream);
+    return launch_heads_lds<16>(a, lds, tiles, wide, stream);
+  }
   if (dtype == ME_BF16 && pieces && (T + 63) / 64 <= 65535) {
     heads_linear_mfma_kernel<<<dim3((unsigned)((N + 15) / 16), (unsigned)((T + 63) / 64), (unsigned)H), dim3(256), 0, stream>>>(a);
   } else {
