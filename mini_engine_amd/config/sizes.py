@@ -120,7 +120,7 @@ def goluzen_config(size: str, layers: int | None = None):
                           "mixer": dict({"heads": Hq, "dim": D, "rot_dim": D // 2, "vdim": D, "kv_rank": 3 * D // 2, "scale": (3 * D // 2) ** -0.5,
                                          "rot": {"dims": D // 2, "base": 1e6, "scaling": {"factor": 4.0, "original": 8192, "fast": 32.0, "slow": 1.0}},
                                          "mask": {"size": 2048}}, **({} if src is None else {"kv_from": src}))}
-    linear = {"type": "gla", "mixer": {"heads": max(1, Hq // 4), "dim": D, "vdim": 2 * D, "tau": 16.0, "decay_rank": 8 if small else 16}}
+    linear = {"type": "gla", "mixer": {"heads": max(1, Hq // 4), "dim": D, "vdim": 2 * D, "tau": 8.0, "decay_rank": 8 if small else 16}}
     moe = {"kind": "moe", "expert": {"ff": max(8, I // 8)}, "shared": {"ff": max(8, I // 2)},
            "router": {"experts": 32, "top": 4, "scale": 2.5, "groups": {"count": 4, "keep": 2}}}
     out, last_own = [], None

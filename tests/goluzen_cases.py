@@ -106,6 +106,21 @@ CONFIGS = {
         _with(_gla(1, 16, 16, 1.0, 4), _moe(16, 2, 1)),
         _with(_attention(2, 2, 8, 8, 1.8, 4, 100.0, None, 5), None),
     ]),
+    # a width in whole 16-byte pieces around sizes that are not (the kernels' vector paths beside their scalar ones in one
+    # model); two latents of different sizes, each with a reader; two experts kept of two
+    "mid": _model(120, 64, 1e-5, [
+        _with(_latent(3, 10, 6, 14, 22, 1.0, 700.0, (3.0, 24, 6.0, 1.0), 12), _moe(24, 2, 2, 1.1, None, 16)),
+        _with(_latent(2, 16, 8, 8, 24, 0.9, 900.0, None, 7), _dense(72)),
+        _with(_gla(3, 6, 10, 5.0, 3), _moe(12, 9, 4, 0.9, (3, 2), 28)),
+        _with(_latent(5, 10, 6, 6, 22, 1.2, 700.0, (3.0, 24, 6.0, 1.0), 30, src=0), None),
+        _with(_attention(6, 2, 12, 10, 1.3, 6, 700.0, 2.5, 9, 2, 7.0), _dense(40)),
+        _with(_latent(1, 16, 8, 24, 24, 1.1, 900.0, None, None, src=1), _moe(16, 4, 2, 1.3, (2, 1))),
+    ], 3.0),
+    # nothing but linear attention: a model without any pages
+    "flat": _model(50, 24, 1e-5, [
+        _with(_gla(2, 4, 6, 2.0, 3), _dense(32)),
+        _with(_gla(1, 12, 8, 6.0, 4), None),
+    ]),
     # long windows with few kept positions: keys hundreds of positions back
     "far": _model(80, 32, 1e-5, [
         _with(_attention(2, 1, 16, 16, 1.5, 8, 50000.0, 4.0, 300, 4, 20.0), _dense(48)),
@@ -117,7 +132,7 @@ CONFIGS = {
     "real": _model(2048, 1024, 1e-6, [
         _with(_attention(16, 8, 128, 128, 128 ** -0.5 * 4, 64, 1e6, 4.0, 256, 16, 50.0), _dense(3072)),
         _with(_latent(16, 128, 64, 128, 192, 192 ** -0.5 * 2, 1e6, (4.0, 8192, 32.0, 1.0), 384), _moe(384, 8, 8, 0.6, (2, 2), 1536)),
-        _with(_gla(4, 128, 256, 16.0, 16), _moe(384, 8, 8, 0.6, (2, 2), 1536)),
+        _with(_gla(4, 128, 256, 8.0, 16), _moe(384, 8, 8, 0.6, (2, 2), 1536)),
         _with(_latent(16, 128, 64, 128, 192, 192 ** -0.5 * 2, 1e6, (4.0, 8192, 32.0, 1.0), 128, src=1), _moe(384, 8, 8, 0.6, None, 1536)),
     ], 8.0),
     # the same with 4 of 32 experts per token: a token whose choice hangs on two scores closer than bfloat16's rounding of the
@@ -125,12 +140,12 @@ CONFIGS = {
     "routed": _model(2048, 1024, 1e-6, [
         _with(_attention(16, 8, 128, 128, 128 ** -0.5 * 4, 64, 1e6, 4.0, 256, 16, 50.0), _dense(3072)),
         _with(_latent(16, 128, 64, 128, 192, 192 ** -0.5 * 2, 1e6, (4.0, 8192, 32.0, 1.0), 384), _moe(384, 32, 4, 2.5, (4, 2), 1536)),
-        _with(_gla(4, 128, 256, 16.0, 16), _moe(384, 32, 4, 2.5, (4, 2), 1536)),
+        _with(_gla(4, 128, 256, 8.0, 16), _moe(384, 32, 4, 2.5, (4, 2), 1536)),
     ], 8.0),
 }
-SEEDS = {"mix": 31, "odd": 32, "one": 33, "far": 34, "real": 35, "routed": 36}
-PAGE = {"mix": 16, "odd": 8, "one": 4, "far": 16, "real": 16, "routed": 16}
-SMALL = ("mix", "odd", "one")
+SEEDS = {"mix": 31, "odd": 32, "one": 33, "far": 34, "real": 35, "routed": 36, "mid": 37, "flat": 38}
+PAGE = {"mix": 16, "odd": 8, "one": 4, "far": 16, "real": 16, "routed": 16, "mid": 32, "flat": 16}
+SMALL = ("mix", "odd", "one", "mid", "flat")
 
 
 def make_folder(name: str, path: str) -> str:
