@@ -1348,7 +1348,9 @@ constexpr bool DECODE_STREAMS = ME_DECODE_STREAMS != 0;
 // (The values of both ahead as well need 197 registers, which leaves two workgroups to a compute unit instead of
 // three.)
 template <bool PROLOGUE, bool AHEAD = false>
-__global__ void __launch_bounds__(256, 3) attn_decode_kernel(AttnArgs a) {
+// Three workgroups to a compute unit (170 registers a lane) up to head size 128; a block's key and value operands of a larger
+// head need more than that, and two (256 registers) or one workgroup keep them out of scratch memory.
+__global__ void __launch_bounds__(256, HD <= 128 ? 3 : (HD <= 256 ? 2 : 1)) attn_decode_kernel(AttnArgs a) {
   extern __shared__ float lds[];  // [4 waves][cols][HD + 2]; PROLOGUE: then bfloat16 [cols + 2][HD]
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int n = lane & 15, g = lane >> 4;
@@ -1679,11 +1681,20 @@ extern "C" int me_attn_prefill(const void* q, int64_t q_stride, void* out, int64
     a.seq_of_token = seq_of_token; a.seq_base = seq_base;
   }
   const dim3 grid((unsigned)(tiles * Hkv), 1, a.max_segs);
-  // Keys and values through LDS where the two buffers fit (head sizes up to 128); the caller cuts
-  // long key ranges so that there are workgroups enough for that form to pay (with one workgroup
-  // per CU its waves have no others to fill their waits at the barriers).
+  // Keys and values through LDS where the two buffers of two workgroups fit a compute unit's 160 KB (head sizes up
+  // to 272); the caller cuts long key ranges so that there are workgroups enough for that form to pay (with one
+  // workgroup per CU its waves have no others to fill their waits at the barriers).
   // shared: 0 never, otherwise wherever it fits.
-  const bool through_lds = 2 * PF_BUF <= 65536 && shared != 0;
+  const bool through_lds = 2 * PF_BUF <= 80 * 1024 && shared != 0;
+  if (through_lds && 2 * PF_BUF > 64 * 1024) {          // more LDS than a kernel may have unasked
+    static bool allowed = false;
+    if (!allowed) {
+      hipError_t e1 = hipFuncSetAttribute((const void*)attn_prefill_shared_kernel<1>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * PF_BUF);
+      hipError_t e2 = hipFuncSetAttribute((const void*)attn_prefill_shared_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, 2 * PF_BUF);
+      ME_CHECK(e1 == hipSuccess && e2 == hipSuccess, "attention: cannot get %d bytes of LDS", 2 * PF_BUF);
+      allowed = true;
+    }
+  }
 #if ME_HEAD_DIM == 128
   // shared: 1 the memory system fills LDS where the kernel for that applies, 2 always through registers.
   // waves: 3 asks for three waves to a SIMD (168 registers each) instead of two, with two column tiles; the

@@ -436,6 +436,8 @@ class HipBackend:
             num_decodes = 0
         if num_decodes > 0:
             part_size, num_parts = decode_partitions(num_decodes, Hq, Hkv, max_decode_context, even_contexts)
+            if D > 128:
+                part_size, num_parts = wide_head_partitions(part_size, num_parts, num_decodes * Hkv * ((Hq // Hkv + 15) // 16), max_decode_context)
             scratch = _scratch(num_decodes * Hq * num_parts * (D + 2), q.device) if num_parts > 1 else None
             lib.call("me_attn_decode", q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), k_cache.data_ptr(),
                      v_cache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(),
@@ -1512,6 +1514,18 @@ def decode_partitions(num_seqs: int, Hq: int, Hkv: int, max_context: int, even: 
     want = min(64, want)
     part = max(128, -(-(-(-ctx // want)) // 128) * 128)
     parts = max(1, -(-ctx // part))
+    return part, parts
+
+
+def wide_head_partitions(part: int, parts: int, base: int, max_context: int) -> tuple:
+    """`decode_partitions` for head sizes above 128: the decode kernel then has two workgroups to a compute unit (its
+    operands of a block need more registers than three leave) and a block costs it more, so more than one round of
+    workgroups does not pay: partitions are doubled while more than one workgroup per compute unit remains (64 requests
+    of 2,048 keys under one key/value head of 256: 8 partitions of 256 keys 60 us, 4 of 512 34 us; 8 requests keep
+    their 16 partitions of 128 keys, 17 us, where 8 of 256 take 25)."""
+    while parts > 1 and base * parts > _COMPUTE_UNITS and part < _DECODE_MAX_PARTITION:
+        part *= 2
+        parts = max(1, -(-max(1, max_context) // part))
     return part, parts
 
 

@@ -243,3 +243,13 @@ def test_decode_partitions_always_fit_the_kernel():
         assert part % 32 == 0 and part >= 128 and parts >= 1, (S, Hq, Hkv, ctx, even, part, parts)
         assert part * parts >= ctx and part * (parts - 1) < ctx, (S, Hq, Hkv, ctx, even, part, parts)
         assert parts <= 64, (S, Hq, Hkv, ctx, even, part, parts)
+
+
+def test_partitions_for_wide_heads():
+    # more than a workgroup per compute unit: doubled until one round is left; fewer: as they are
+    assert ops.wide_head_partitions(256, 8, 64, 2048) == (512, 4) and ops.wide_head_partitions(128, 16, 8, 2048) == (128, 16)
+    assert ops.wide_head_partitions(128, 16, 1, 2048) == (128, 16) and ops.wide_head_partitions(2048, 1, 512, 2048) == (2048, 1)
+    for base in (1, 3, 64, 100, 500):
+        for ctx in (1, 129, 2048, 5000, 70000):
+            part, parts = ops.wide_head_partitions(*ops.decode_partitions(base, 16, 1, ctx), base, ctx)
+            assert part * parts >= ctx and part * (parts - 1) < ctx and part % 32 == 0
